@@ -1,0 +1,160 @@
+/* llmq.h - C ABI of libllmq_gfx950.so: the quantized-linear hot path of LLMQRT as
+ * hand-written HIP kernels for AMD Instinct MI355X (gfx950 / CDNA4).
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer unless its comment says "host".
+ *  - The caller owns every buffer (inputs, outputs, workspaces); the library allocates
+ *    nothing, keeps no state between calls, never synchronises with the host and launches
+ *    on the stream it is given (0 = the null stream).  Calls are asynchronous.
+ *  - Matrices are row-major; `ld*` is the row stride in ELEMENTS.
+ *  - Return value: LLMQ_OK (0) or a negative llmq_status; llmq_status_string() names it.
+ *  - Paths below are relative to the reference's runtime/ directory.
+ */
+#ifndef LLMQ_H_
+#define LLMQ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* llmq_stream_t; /* a hipStream_t */
+
+typedef enum {
+    LLMQ_OK = 0,
+    LLMQ_ERR_NULL = -1,      /* a required pointer is NULL */
+    LLMQ_ERR_DTYPE = -2,     /* unsupported dtype / format selector */
+    LLMQ_ERR_SHAPE = -3,     /* negative size, stride smaller than the row, unsupported alignment */
+    LLMQ_ERR_WORKSPACE = -4, /* workspace missing or too small */
+    LLMQ_ERR_LAUNCH = -5,    /* the HIP runtime refused the launch (hipGetLastError) */
+    LLMQ_ERR_ALIGN = -6      /* a pointer is not 16-byte aligned */
+} llmq_status;
+
+typedef enum { LLMQ_BF16 = 0, LLMQ_F16 = 1, LLMQ_F32 = 2 } llmq_dtype;
+typedef enum { LLMQ_E4M3 = 0, LLMQ_E5M2 = 1 } llmq_fp8_format; /* OCP e4m3fn / e5m2 */
+
+int llmq_abi_version(void);
+const char* llmq_status_string(int status); /* host pointer to a static string */
+
+/* ------------------------------------------------------------------------------------
+ * Activation quantizers.  The reference runs each of these as 5-7 eager torch ops.
+ * All arithmetic follows the reference bit for bit: it is carried out in the dtype of x
+ * (the clamp bound, the scale and the quotient x/scale are each rounded to x_dtype).
+ * x: [M, K] bf16/f16, K % 8 == 0, ldx % 8 == 0, 16-byte aligned.
+ * ------------------------------------------------------------------------------------ */
+
+/* Replaces quantize_activation_per_token_absmax, nn_models/modules/linear/linear_sq.py:55-65.
+ * q: int8 [M, K] contiguous.  scale: [M] in x_dtype (scale_dtype == x_dtype) or fp32
+ * (scale_dtype == LLMQ_F32, the same value widened - what the GEMM epilogue consumes). */
+int llmq_quant_i8_per_token(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                            int8_t* q, void* scale, int scale_dtype, llmq_stream_t stream);
+
+/* Replaces quantize_activation_per_tensor_absmax, linear_sq.py:44-53.  scale: one element.
+ * workspace: >= llmq_quant_workspace_bytes() bytes, contents irrelevant on entry. */
+int llmq_quant_i8_per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                             int8_t* q, void* scale, int scale_dtype,
+                             void* workspace, size_t workspace_bytes, llmq_stream_t stream);
+
+/* Replaces per_token_quantize, nn_models/modules/linear/linear_fp8.py:40-63.
+ * q: e4m3fn bytes [M, K] contiguous; scale: fp32 [M]. */
+int llmq_quant_fp8_per_token(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                             uint8_t* q, float* scale, llmq_stream_t stream);
+
+/* Replaces per_tensor_quantize, linear_fp8.py:11-32.  scale: fp32, one element. */
+int llmq_quant_fp8_per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                              uint8_t* q, float* scale,
+                              void* workspace, size_t workspace_bytes, llmq_stream_t stream);
+
+/* Replaces static_per_tensor_quantize, linear_fp8.py:34-37.  scale: fp32 device scalar; the
+ * quotient is formed in fp32 (tensor / fp32 tensor promotes) when scale_is_f32_tensor != 0,
+ * else the scalar is first rounded to x_dtype and the quotient rounded to x_dtype. */
+int llmq_quant_fp8_static(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                          uint8_t* q, const float* scale, int scale_is_f32_tensor,
+                          llmq_stream_t stream);
+
+size_t llmq_quant_workspace_bytes(void);
+
+/* ------------------------------------------------------------------------------------
+ * W8A8 int8 GEMM.  Replaces w8a8_int8_linear_bbf16_obf16_per_tensor
+ * (csrc/smoothquant/sq_gemm.cu:36-160, bound at csrc/bindings.cpp:10-11) and implements the
+ * per-token x per-channel op the reference only declares
+ * (w8a8_int8_linear_bbf16_obf16_per_channel, csrc/smoothquant/sq_gemm.h:19-24).
+ *
+ *   acc[m,n] = sum_k A[m,k] * B[n,k]                         (int32, exact)
+ *   out[m,n] = out_dtype( f(acc[m,n]) )
+ *     a_scale == NULL && w_scale == NULL:  f = alpha' * acc + beta * bias[n]
+ *     otherwise:                           f = (acc * sa[m]) * sw[n] * alpha' + beta * bias[n]
+ *   alpha' = alpha * (alpha_dev ? *alpha_dev : 1); sa/sw default to 1 when NULL; bias may be NULL.
+ *
+ * A: int8 [M,K] (lda >= K).  B: int8 [N,K] row-major (ldb >= K) - the reference passes the
+ * same memory as a [K,N] view with stride (1,K).  K % 16 == 0, lda % 16 == 0, ldb % 16 == 0.
+ * a_scale: fp32 [M]; w_scale: fp32 [N]; alpha_dev: fp32 device scalar (removes the
+ * reference's .item() host syncs, linear_sq.py:127); bias: [N] of bias_dtype (bf16/f16/f32).
+ * out: [M,N] bf16/f16 (ldo >= N).  acc_dump: optional int32 [M,N] contiguous that receives
+ * the raw accumulators (parity checks).  workspace: >= llmq_gemm_workspace_bytes(M,N,K)
+ * bytes (may be NULL when that is 0); contents irrelevant on entry.
+ * ------------------------------------------------------------------------------------ */
+int llmq_gemm_w8a8(const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb,
+                   const float* a_scale, const float* w_scale,
+                   float alpha, const float* alpha_dev,
+                   const void* bias, int bias_dtype, float beta,
+                   void* out, int out_dtype, int64_t ldo,
+                   int64_t M, int64_t N, int64_t K,
+                   int32_t* acc_dump, void* workspace, size_t workspace_bytes,
+                   llmq_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * FP8 scaled GEMM.  Replaces f8f8bf16_rowwise (csrc/fp8/sm89_fp8_rowwise_fbgemm.cu:582-606,
+ * bound as cutlass_f8f8bf16_rowwise_sm89 at csrc/bindings.cpp:13) and f8f8bf16_tensorwise
+ * (csrc/fp8/sm89_fp8_tensorwise_cutlassgemm.cu:316-334, bound at csrc/bindings.cpp:12).
+ * Same contract as llmq_gemm_w8a8 with fp32 accumulation of exact fp8 products:
+ * A: fp8 bytes [M,K] in a_format (e4m3fn or e5m2); B: e4m3fn bytes [N,K].
+ * acc_dump: optional fp32 [M,N].
+ * ------------------------------------------------------------------------------------ */
+int llmq_gemm_fp8(const uint8_t* A, int a_format, int64_t lda, const uint8_t* B, int64_t ldb,
+                  const float* a_scale, const float* w_scale,
+                  float alpha, const float* alpha_dev,
+                  const void* bias, int bias_dtype, float beta,
+                  void* out, int out_dtype, int64_t ldo,
+                  int64_t M, int64_t N, int64_t K,
+                  float* acc_dump, void* workspace, size_t workspace_bytes,
+                  llmq_stream_t stream);
+
+size_t llmq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/* Tuning / test hook with no counterpart in the reference: force tile configuration `cfg`
+ * (0 .. llmq_gemm_num_configs()-1) and K split `splits` for every later GEMM call of this
+ * process; cfg < 0 restores the built-in heuristic.  Process-global, not thread-safe. */
+int llmq_gemm_force_plan(int cfg, int splits);
+int llmq_gemm_num_configs(void);
+
+/* ------------------------------------------------------------------------------------
+ * AWQ W4A16.  Replaces awq_gemm_triton / awq_dequantize_triton
+ * (triton_kernels/awq_kernels.py:328-378 / :273-320).
+ * qweight: int32 [K, N/8], nibble i of a word = logical column 8c + {0,2,4,6,1,3,5,7}[i]
+ * (nn_models/modules/linear/linear_awq.py:192-202); qzeros: int32 [K/G, N/8], same packing;
+ * scales: fp16 [K/G, N].  G (group) divides K, G % 32 == 0; N % 8 == 0.
+ * ------------------------------------------------------------------------------------ */
+
+/* out[m,n] = fp16( sum_k x[m,k] * fp16((q[k,n] - z[k/G,n]) * s[k/G,n]) + bias[n] ), fp32
+ * accumulation in a fixed order (deterministic, unlike the reference's fp16 atomics).
+ * x: fp16 [M,K] (ldx >= K, K % 32 == 0); out: fp16 [M,N] contiguous; bias: fp16 [N] or NULL.
+ * workspace: >= llmq_awq_gemm_workspace_bytes(M,N,K) bytes. */
+int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight, const void* scales,
+                  const int32_t* qzeros, const void* bias, void* out,
+                  int64_t M, int64_t N, int64_t K, int64_t group,
+                  void* workspace, size_t workspace_bytes, llmq_stream_t stream);
+
+size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/* out: fp16 [K, N] contiguous = fp16(q - z) * s, bit-exact with
+ * utils/packing_utils.py:65-80 (dequantize_gemm). */
+int llmq_awq_dequant(const int32_t* qweight, const void* scales, const int32_t* qzeros,
+                     void* out, int64_t K, int64_t N, int64_t group, llmq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLMQ_H_ */

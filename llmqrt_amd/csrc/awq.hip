@@ -1,0 +1,373 @@
+// AWQ W4A16: group-dequant GEMM for decode shapes and the standalone dequantizer.
+//
+// Weight layout (nn_models/modules/linear/linear_awq.py:192-202): qweight int32 [K, N/8];
+// nibble p of a word holds logical column 8c + {0,2,4,6,1,3,5,7}[p], i.e. logical column j is
+// nibble REV[j] with REV = {0,4,1,5,2,6,3,7} (utils/packing_utils.py:5).  qzeros [K/G, N/8]
+// uses the same packing, scales are fp16 [K/G, N].
+//
+// GEMM kernel.  The op is HBM-bound (half a byte per weight), so the only goal is to stream
+// qweight at full rate and keep the unpack cheap enough for the VALU to keep up:
+//   * out^T = W^T x^T on v_mfma_f32_16x16x32_f16: the MFMA "A" rows are 16 output channels,
+//     the "B" columns are up to 16 tokens, both operands want 8 consecutive k per lane.
+//   * A lane loads the words of 8 consecutive k-rows for its word column(s) with plain
+//     coalesced global loads (no LDS): that 8x8 block of nibbles is the A operand of 8 MFMAs,
+//     one per logical column j.  For column j, v_perm_b32 pulls the byte that holds nibble
+//     REV[j] out of two k-adjacent words into the low bytes of the two halves of a register;
+//     (u & 0x000F000F) | 0x64006400 then reads as two fp16 values 1024+q (low nibble) or
+//     (u & 0x00F000F0) | 0x64006400 as 1024+16q (high nibble); one packed add / fma removes
+//     the bias and the zero point exactly, one packed multiply applies the group scale with
+//     the same single fp16 rounding as the reference dequantizer.  ~2 VALU ops per weight.
+//   * fp32 accumulation in the MFMA; the 4 wavefronts of a block split the block's K range and
+//     are summed through LDS in a fixed order; a K split across blocks goes through an fp32
+//     workspace and a finishing kernel, again in a fixed order (results are deterministic).
+#include "llmq_common.h"
+
+namespace llmq {
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+__host__ __device__ constexpr int rev_nibble(int j) { return ((j & 1) << 2) | (j >> 1); }  // {0,4,1,5,2,6,3,7}
+
+template <int V> struct WordVec;
+template <> struct WordVec<1> { typedef uint32_t type; };
+template <> struct WordVec<2> { typedef uint2 type; };
+template <> struct WordVec<4> { typedef uint4 type; };
+
+template <int V> __device__ __forceinline__ uint32_t word_of(const typename WordVec<V>::type& v, int t);
+template <> __device__ __forceinline__ uint32_t word_of<1>(const uint32_t& v, int) { return v; }
+template <> __device__ __forceinline__ uint32_t word_of<2>(const uint2& v, int t) { return t ? v.y : v.x; }
+template <> __device__ __forceinline__ uint32_t word_of<4>(const uint4& v, int t) {
+    return t == 0 ? v.x : (t == 1 ? v.y : (t == 2 ? v.z : v.w));
+}
+
+constexpr int kChunkK = 32;  // k per MFMA step
+constexpr int kBlockWaves = 4;
+
+// V: words (of 8 columns) per lane -> a wavefront covers 128*V output channels.
+// MT: 16-token tiles (M <= 16*MT).
+template <int V, int MT>
+__global__ __launch_bounds__(kBlockWaves * kWave) void awq_gemm_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, const uint32_t* __restrict__ qw,
+    const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qz, const uint16_t* __restrict__ bias,
+    uint16_t* __restrict__ out, float* __restrict__ partials, int M, int N, int K, int G, int chunks_per_block) {
+    typedef typename WordVec<V>::type wvec;
+    constexpr int NACC = MT * V * 8;
+    __shared__ float4 red[NACC * kWave];
+
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int li = lane & 15, kb = lane >> 4;
+    const int Nw = N >> 3;
+    const int cw = blockIdx.x * (16 * V) + V * li;  // first word column of this lane
+    const bool col_ok = cw < Nw;
+    const int cwc = col_ok ? cw : 0;
+
+    const int total_chunks = K / kChunkK;
+    const int cb0 = blockIdx.y * chunks_per_block, cb1 = min(total_chunks, cb0 + chunks_per_block);
+    const int cpw = (cb1 - cb0 + kBlockWaves - 1) / kBlockWaves;
+    const int c0 = cb0 + wave * cpw, c1 = min(cb1, c0 + cpw);
+
+    v4f acc[MT][V][8];
+#pragma unroll
+    for (int a = 0; a < MT; a++)
+#pragma unroll
+        for (int t = 0; t < V; t++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[a][t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    h2 cz[V][8], s2[V][8];  // per-group constants: -(bias+zero) and the scale, both halves equal
+    int cur_g = -1;
+
+    wvec wcur[8], wnext[8];
+    uint4 xcur[MT], xnext[MT];
+    auto load_chunk = [&](int c, wvec* wdst, uint4* xdst) {
+        const int k0 = c * kChunkK + 8 * kb;
+        const uint32_t* wp = qw + (int64_t)k0 * Nw + cwc;
+#pragma unroll
+        for (int r = 0; r < 8; r++) wdst[r] = *reinterpret_cast<const wvec*>(wp + (int64_t)r * Nw);
+#pragma unroll
+        for (int a = 0; a < MT; a++) {
+            const int m = a * 16 + li;
+            xdst[a] = m < M ? *reinterpret_cast<const uint4*>(x + (int64_t)m * ldx + k0) : make_uint4(0, 0, 0, 0);
+        }
+    };
+
+    if (c0 < c1) load_chunk(c0, wcur, xcur);
+    for (int c = c0; c < c1; c++) {
+        if (c + 1 < c1) load_chunk(c + 1, wnext, xnext);
+        const int g = (c * kChunkK) / G;
+        if (g != cur_g) {
+            cur_g = g;
+            const wvec zv = *reinterpret_cast<const wvec*>(qz + (int64_t)g * Nw + cwc);
+#pragma unroll
+            for (int t = 0; t < V; t++) {
+                const uint32_t zw = word_of<V>(zv, t);
+                const uint4 sv = *reinterpret_cast<const uint4*>(scales + (int64_t)g * N + 8 * (cwc + t));
+                const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w};
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    constexpr uint32_t kLoBase = 0xE400u, kHiBase = 0xD400u;  // -(1024), -(64) as fp16 bits
+                    const int p = rev_nibble(j);
+                    const uint32_t z = (zw >> (4 * p)) & 0xFu;
+                    const uint32_t c16 = (p & 1) ? (kHiBase | (z << 4)) : (kLoBase | z);  // -(64+z) / -(1024+z)
+                    cz[t][j] = __builtin_bit_cast(h2, c16 * 0x00010001u);
+                    const uint32_t sh = (j & 1) ? (sw[j >> 1] >> 16) : (sw[j >> 1] & 0xffffu);
+                    s2[t][j] = __builtin_bit_cast(h2, sh * 0x00010001u);
+                }
+            }
+        }
+        h8 xb[MT];
+#pragma unroll
+        for (int a = 0; a < MT; a++) xb[a] = __builtin_bit_cast(h8, xcur[a]);
+#pragma unroll
+        for (int t = 0; t < V; t++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int p = rev_nibble(j);
+                const uint32_t sel = (uint32_t)(p >> 1) | 0x0c00u | ((uint32_t)(4 + (p >> 1)) << 16) | 0x0c000000u;
+                uint32_t ar[4];
+#pragma unroll
+                for (int pr = 0; pr < 4; pr++) {
+                    const uint32_t w0 = word_of<V>(wcur[2 * pr], t), w1 = word_of<V>(wcur[2 * pr + 1], t);
+                    const uint32_t u = __builtin_amdgcn_perm(w1, w0, sel);  // byte0 <- w0, byte2 <- w1
+                    h2 d;
+                    if (p & 1) {
+                        const h2 h = __builtin_bit_cast(h2, (u & 0x00F000F0u) | 0x64006400u);  // 1024 + 16 q
+                        const h2 k16 = {(_Float16)0.0625f, (_Float16)0.0625f};
+                        d = __builtin_elementwise_fma(h, k16, cz[t][j]);                       // q - z, exact
+                    } else {
+                        const h2 h = __builtin_bit_cast(h2, (u & 0x000F000Fu) | 0x64006400u);  // 1024 + q
+                        d = h + cz[t][j];                                                      // q - z, exact
+                    }
+                    ar[pr] = __builtin_bit_cast(uint32_t, d * s2[t][j]);  // fp16((q - z) * s), one rounding
+                }
+                const h8 af = __builtin_bit_cast(h8, v4i{(int)ar[0], (int)ar[1], (int)ar[2], (int)ar[3]});
+#pragma unroll
+                for (int a = 0; a < MT; a++)
+                    acc[a][t][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, xb[a], acc[a][t][j], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 8; r++) wcur[r] = wnext[r];
+#pragma unroll
+        for (int a = 0; a < MT; a++) xcur[a] = xnext[a];
+    }
+
+    // ---- sum the 4 wavefronts in wave order through LDS ---------------------------------------
+    for (int src = 1; src < kBlockWaves; src++) {
+        __syncthreads();
+        if (wave == src) {
+#pragma unroll
+            for (int a = 0; a < MT; a++)
+#pragma unroll
+                for (int t = 0; t < V; t++)
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const v4f v = acc[a][t][j];
+                        red[((a * V + t) * 8 + j) * kWave + lane] = make_float4(v[0], v[1], v[2], v[3]);
+                    }
+        }
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int a = 0; a < MT; a++)
+#pragma unroll
+                for (int t = 0; t < V; t++)
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const float4 v = red[((a * V + t) * 8 + j) * kWave + lane];
+                        acc[a][t][j] += v4f{v.x, v.y, v.z, v.w};
+                    }
+        }
+    }
+    if (wave != 0) return;
+
+    // ---- store: lane (token li, quarter kb) holds rows 4*kb + r of every MFMA tile, i.e. the 8
+    // consecutive channels 8*(cw_tile + V*(4*kb + r) + t) + j, j = 0..7 ------------------------
+    const bool split = gridDim.y > 1;
+#pragma unroll
+    for (int a = 0; a < MT; a++) {
+        const int m = a * 16 + li;
+        if (m >= M) continue;
+#pragma unroll
+        for (int t = 0; t < V; t++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int wcol = blockIdx.x * (16 * V) + V * (4 * kb + r) + t;
+                if (wcol >= Nw) continue;
+                const int n = 8 * wcol;
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = acc[a][t][j][r];
+                if (split) {
+                    float4* dst = reinterpret_cast<float4*>(partials + ((int64_t)blockIdx.y * M + m) * N + n);
+                    dst[0] = make_float4(v[0], v[1], v[2], v[3]);
+                    dst[1] = make_float4(v[4], v[5], v[6], v[7]);
+                } else {
+                    uint32_t o[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float lo = v[2 * j], hi = v[2 * j + 1];
+                        if (bias) {
+                            lo = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(lo)) + Lo<LLMQ_F16>::to_f32(bias[n + 2 * j]);
+                            hi = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(hi)) + Lo<LLMQ_F16>::to_f32(bias[n + 2 * j + 1]);
+                        }
+                        o[j] = (uint32_t)Lo<LLMQ_F16>::from_f32(lo) | ((uint32_t)Lo<LLMQ_F16>::from_f32(hi) << 16);
+                    }
+                    *reinterpret_cast<uint4*>(out + (int64_t)m * N + n) = make_uint4(o[0], o[1], o[2], o[3]);
+                }
+            }
+        }
+    }
+}
+
+// Cross-block split-K finish: sum partials in split order, round to fp16, add bias.
+__global__ __launch_bounds__(256) void awq_finish_kernel(const float* __restrict__ partials, int splits, int64_t total,
+                                                         int N, const uint16_t* __restrict__ bias,
+                                                         uint16_t* __restrict__ out) {
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        float s = 0.f;
+        for (int i = 0; i < splits; i++) s += partials[i * total + idx];
+        if (bias) s = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(s)) + Lo<LLMQ_F16>::to_f32(bias[idx % N]);
+        out[idx] = Lo<LLMQ_F16>::from_f32(s);
+    }
+}
+
+// Standalone dequantizer: one thread per packed word -> 8 fp16 (16-byte store).
+__global__ __launch_bounds__(256) void awq_dequant_kernel(const uint32_t* __restrict__ qw,
+                                                          const uint16_t* __restrict__ scales,
+                                                          const uint32_t* __restrict__ qz, uint16_t* __restrict__ out,
+                                                          int64_t K, int Nw, int G) {
+    const int64_t total = K * Nw;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t k = idx / Nw;
+        const int c = (int)(idx - k * Nw);
+        const int64_t g = k / G;
+        const uint32_t w = qw[idx], z = qz[g * Nw + c];
+        const uint4 sv = *reinterpret_cast<const uint4*>(scales + (g * Nw + c) * 8);
+        const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int j2 = 0; j2 < 4; j2++) {
+            uint32_t pair = 0;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int j = 2 * j2 + h, sh = 4 * rev_nibble(j);
+                const int d = (int)((w >> sh) & 0xFu) - (int)((z >> sh) & 0xFu);
+                const _Float16 s = __builtin_bit_cast(_Float16, (uint16_t)(h ? (sw[j2] >> 16) : (sw[j2] & 0xffffu)));
+                const _Float16 v = (_Float16)d * s;  // exact difference, one fp16 RNE multiply
+                pair |= (uint32_t)__builtin_bit_cast(uint16_t, v) << (16 * h);
+            }
+            o[j2] = pair;
+        }
+        *reinterpret_cast<uint4*>(out + idx * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+struct AwqPlan { int v, mt, splits, chunks_per_block; };
+
+inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+AwqPlan make_awq_plan(int64_t M, int64_t N, int64_t K) {
+    AwqPlan p;
+    p.mt = cdiv(M, 16);
+    const int Nw = (int)(N / 8);
+    p.v = (p.mt == 1 && Nw % 2 == 0 && N >= 16384) ? 2 : 1;
+    const int ntiles = cdiv(Nw, 16 * p.v);
+    const int chunks = (int)(K / kChunkK);
+    // aim at ~2 blocks per CU; every wavefront should keep at least 4 chunks
+    int splits = cdiv(512, ntiles);
+    const int max_splits = chunks / (4 * kBlockWaves) > 0 ? chunks / (4 * kBlockWaves) : 1;
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    p.chunks_per_block = cdiv(chunks, splits);
+    p.splits = cdiv(chunks, p.chunks_per_block);
+    return p;
+}
+
+template <int V, int MT>
+void launch_awq(const AwqPlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
+                const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K, int G,
+                hipStream_t st) {
+    const int ntiles = cdiv(N / 8, 16 * V);
+    hipLaunchKernelGGL((awq_gemm_kernel<V, MT>), dim3(ntiles, p.splits), dim3(kBlockWaves * kWave), 0, st, x, ldx, qw,
+                       scales, qz, bias, out, ws, M, N, K, G, p.chunks_per_block);
+}
+
+}  // namespace
+}  // namespace llmq
+
+using namespace llmq;
+
+extern "C" size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    size_t total = 0;
+    for (int64_t m0 = 0; m0 < M; m0 += 64) {
+        const int64_t mm = M - m0 < 64 ? M - m0 : 64;
+        const AwqPlan p = make_awq_plan(mm, N, K);
+        const size_t need = p.splits > 1 ? (size_t)p.splits * mm * N * sizeof(float) : 0;
+        if (need > total) total = need;
+    }
+    return total;
+}
+
+extern "C" int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight, const void* scales,
+                             const int32_t* qzeros, const void* bias, void* out, int64_t M, int64_t N, int64_t K,
+                             int64_t group, void* workspace, size_t workspace_bytes, llmq_stream_t stream) {
+    if (M < 0 || N < 0 || K < 0) return LLMQ_ERR_SHAPE;
+    if (M == 0 || N == 0) return LLMQ_OK;
+    if (!x || !qweight || !scales || !qzeros || !out) return LLMQ_ERR_NULL;
+    if (K == 0 || (K % kChunkK) || (N & 7) || group <= 0 || (K % group) || (group % kChunkK) || ldx < K || (ldx & 7))
+        return LLMQ_ERR_SHAPE;
+    if (N > 0x7fffffffLL || K > 0x7fffffffLL || M > 0x7fffffffLL) return LLMQ_ERR_SHAPE;
+    if (!aligned16(x) || !aligned16(scales) || !aligned16(out) || (reinterpret_cast<uintptr_t>(qweight) & 15u) ||
+        (reinterpret_cast<uintptr_t>(qzeros) & 15u))
+        return LLMQ_ERR_ALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    // tokens are processed in slabs of at most 64 rows (4 MFMA token tiles per weight pass)
+    for (int64_t m0 = 0; m0 < M; m0 += 64) {
+        const int mm = (int)(M - m0 < 64 ? M - m0 : 64);
+        const AwqPlan p = make_awq_plan(mm, N, K);
+        float* ws = (float*)workspace;
+        if (p.splits > 1 && (!ws || workspace_bytes < (size_t)p.splits * mm * N * sizeof(float)))
+            return LLMQ_ERR_WORKSPACE;
+        const uint16_t* xs = (const uint16_t*)x + m0 * ldx;
+        uint16_t* os = (uint16_t*)out + m0 * N;
+        const uint32_t* qw = (const uint32_t*)qweight;
+        const uint32_t* qz = (const uint32_t*)qzeros;
+        const uint16_t* sc = (const uint16_t*)scales;
+        const uint16_t* bs = (const uint16_t*)bias;
+        const int Ni = (int)N, Ki = (int)K, Gi = (int)group;
+        if (p.v == 2) launch_awq<2, 1>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
+        else if (p.mt == 1) launch_awq<1, 1>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
+        else if (p.mt == 2) launch_awq<1, 2>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
+        else launch_awq<1, 4>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
+        if (launch_status() != LLMQ_OK) return LLMQ_ERR_LAUNCH;
+        if (p.splits > 1) {
+            const int64_t total = (int64_t)mm * N;
+            const int blocks = (int)((total + 255) / 256 < 2048 ? (total + 255) / 256 : 2048);
+            hipLaunchKernelGGL(awq_finish_kernel, dim3(blocks), dim3(256), 0, st, ws, p.splits, total, Ni, bs, os);
+            if (launch_status() != LLMQ_OK) return LLMQ_ERR_LAUNCH;
+        }
+    }
+    return LLMQ_OK;
+}
+
+extern "C" int llmq_awq_dequant(const int32_t* qweight, const void* scales, const int32_t* qzeros, void* out,
+                                int64_t K, int64_t N, int64_t group, llmq_stream_t stream) {
+    if (K < 0 || N < 0) return LLMQ_ERR_SHAPE;
+    if (K == 0 || N == 0) return LLMQ_OK;
+    if (!qweight || !scales || !qzeros || !out) return LLMQ_ERR_NULL;
+    if ((N & 7) || group <= 0 || (K % group) || N > 0x7fffffffLL) return LLMQ_ERR_SHAPE;
+    if (!aligned16(scales) || !aligned16(out)) return LLMQ_ERR_ALIGN;
+    const int64_t total = K * (N / 8);
+    const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+    hipLaunchKernelGGL(awq_dequant_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const uint32_t*)qweight,
+                       (const uint16_t*)scales, (const uint32_t*)qzeros, (uint16_t*)out, K, (int)(N / 8), (int)group);
+    return launch_status();
+}

@@ -1,0 +1,428 @@
+// W8A8 int8 and FP8 (OCP e4m3fn / e5m2) GEMMs on the gfx950 matrix cores.
+//
+//   acc[m,n] = sum_k A[m,k] * B[n,k]        A: [M,K] row-major, B: [N,K] row-major
+//
+// Both operands are K-contiguous, which is exactly what an MFMA lane wants (each lane feeds
+// 16 or 32 consecutive K-bytes of one row), so tiles move global -> LDS -> registers as
+// 16-byte chunks and nothing is ever transposed.
+//
+// Kernel shape (template GemmCfg): a block of WM x WN wavefronts owns a BM x BN output tile
+// and walks K in BK-byte steps through a double-buffered LDS ring; each wavefront owns a
+// (BM/WM) x (BN/WN) sub-tile made of 32x32 MFMA tiles:
+//   int8: v_mfma_i32_32x32x32_i8      (16 K-bytes per lane per operand, 8 passes)
+//   fp8 : v_mfma_f32_32x32x64_f8f6f4  (32 K-bytes per lane per operand, 16 passes; the
+//         legacy v_mfma_f32_32x32x16_fp8_fp8 runs at half that rate on gfx950)
+// LDS rows are BK bytes; the 16-byte chunk index is XOR-swizzled with the row so that the
+// ds_read_b128 of 16 consecutive rows hits every bank exactly once.
+// The flat block id is first remapped so that each of the 8 XCDs (private L2 each) gets a
+// contiguous range of tiles, then walked in groups of GROUP_M tile-rows for L2 reuse.
+// Split-K (gridDim.y > 1) writes raw accumulators to a workspace; a second kernel reduces
+// them in a fixed order (deterministic) and applies the epilogue.
+#include <algorithm>
+#include <type_traits>
+
+#include "llmq_common.h"
+
+namespace llmq {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kNumXcd = 8;
+constexpr int kGroupM = 8;
+
+struct Epilogue {
+    const float* a_scale;   // [M] or null
+    const float* w_scale;   // [N] or null
+    const float* alpha_dev; // device scalar or null
+    const void* bias;       // [N] or null
+    float alpha, beta;
+    int bias_dtype, out_dtype;
+};
+
+__device__ __forceinline__ float epi_value(float acc, float sa, float sw, float alpha, float bb) {
+    return fmaf(alpha, (acc * sa) * sw, bb);
+}
+__device__ __forceinline__ uint16_t to_out(float v, int out_dtype) {
+    return out_dtype == LLMQ_BF16 ? Lo<LLMQ_BF16>::from_f32(v) : Lo<LLMQ_F16>::from_f32(v);
+}
+
+template <int BM_, int BN_, int BK_, int WM_, int WN_, bool FP8_, int AFMT_ = 0>
+struct GemmCfg {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+    static constexpr bool FP8 = FP8_;
+    static constexpr int AFMT = AFMT_;                 // fp8 A format selector: 0 e4m3, 1 e5m2
+    static constexpr int NT = WM * WN * kWave;
+    static constexpr int WTM = BM / WM, WTN = BN / WN; // wavefront tile
+    static constexpr int TM = WTM / 32, TN = WTN / 32; // MFMA tiles per wavefront
+    static constexpr int CPR = BK / 16;                // 16-byte chunks per LDS row
+    static constexpr int ROWS_PER_LINE = 16 / CPR;     // rows per 256-byte bank line
+    static constexpr int KB = FP8 ? 64 : 32;           // K-bytes one MFMA consumes
+    static constexpr int KSUB = BK / KB;
+    static constexpr int A_LOADS = BM * CPR / NT, B_LOADS = BN * CPR / NT;
+    static constexpr int STAGE_CHUNKS = (BM + BN) * CPR;
+    static constexpr size_t LDS_BYTES = 2u * STAGE_CHUNKS * 16u;
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be 32-aligned");
+    static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "tile must split evenly over threads");
+    static_assert(CPR == 4 || CPR == 8, "BK must be 64 or 128");
+};
+
+template <int CPR>
+__device__ __forceinline__ int lds_chunk(int row, int c) {
+    return row * CPR + (c ^ ((row / (16 / CPR)) & (CPR - 1)));
+}
+
+// flat block id -> (tile_m, tile_n): XCD-contiguous ranges, then GROUP_M-row swizzle
+__device__ __forceinline__ void tile_coords(int bid, int nblk, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int q = nblk / kNumXcd, r = nblk % kNumXcd;
+    const int xcd = bid % kNumXcd, local = bid / kNumXcd;
+    const int pid = xcd < r ? xcd * (q + 1) + local : r * (q + 1) + (xcd - r) * q + local;
+    const int width = kGroupM * tiles_n;
+    const int group = pid / width, first_m = group * kGroupM;
+    const int gsize = min(tiles_m - first_m, kGroupM);
+    tm = first_m + (pid % width) % gsize;
+    tn = (pid % width) / gsize;
+}
+
+template <class C>
+__global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
+    const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
+    int M, int N, int K, int k_per_split, Epilogue ep, void* __restrict__ out, int64_t ldo,
+    void* __restrict__ acc_dump, void* __restrict__ partials) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem_raw[];
+    uint4* lds = reinterpret_cast<uint4*>(smem_raw);
+    using acc_t = typename std::conditional<C::FP8, v16f, v16i>::type;
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int wm = wave / C::WN, wn = wave % C::WN;
+    const int tiles_m = (M + C::BM - 1) / C::BM, tiles_n = (N + C::BN - 1) / C::BN;
+    int tile_m, tile_n;
+    tile_coords(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * C::BM, n0 = tile_n * C::BN;
+    const int k_begin = blockIdx.y * k_per_split;
+    const int k_end = min(K, k_begin + k_per_split);
+    const int ktiles = (k_end - k_begin + C::BK - 1) / C::BK;
+
+    // ---- global -> register staging.  Slot i of a thread is row (tid / CPR) + i * ROWS_STEP at
+    // chunk tid % CPR: the chunk (hence the LDS swizzle) is the same for all of a thread's slots.
+    constexpr int ROWS_STEP = C::NT / C::CPR;
+    static_assert(ROWS_STEP % 16 == 0, "row step must keep the swizzle phase");
+    const int ld_row = tid / C::CPR, ld_c = tid % C::CPR;
+    const uint8_t* a_base = A + (int64_t)m0 * lda + k_begin + ld_c * 16;
+    const uint8_t* b_base = B + (int64_t)n0 * ldb + k_begin + ld_c * 16;
+    int a_off[C::A_LOADS], b_off[C::B_LOADS];  // byte offsets of the (clamped) rows inside the tile
+#pragma unroll
+    for (int i = 0; i < C::A_LOADS; i++) a_off[i] = min(ld_row + i * ROWS_STEP, M - 1 - m0) * (int)lda;
+#pragma unroll
+    for (int i = 0; i < C::B_LOADS; i++) b_off[i] = min(ld_row + i * ROWS_STEP, N - 1 - n0) * (int)ldb;
+    const int st_a = lds_chunk<C::CPR>(ld_row, ld_c);
+    const int st_b = C::BM * C::CPR + st_a;
+    uint4 a_reg[C::A_LOADS], b_reg[C::B_LOADS];
+    auto load_tile = [&](int kt) {
+        const int koff = kt * C::BK;
+        const bool ok = ld_c * 16 < k_end - k_begin - koff;  // chunk inside this split's K range
+#pragma unroll
+        for (int i = 0; i < C::A_LOADS; i++)
+            a_reg[i] = ok ? *reinterpret_cast<const uint4*>(a_base + a_off[i] + koff) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < C::B_LOADS; i++)
+            b_reg[i] = ok ? *reinterpret_cast<const uint4*>(b_base + b_off[i] + koff) : make_uint4(0, 0, 0, 0);
+    };
+    auto store_tile = [&](int stage) {
+        uint4* s = lds + stage * C::STAGE_CHUNKS;
+#pragma unroll
+        for (int i = 0; i < C::A_LOADS; i++) s[st_a + i * ROWS_STEP * C::CPR] = a_reg[i];
+#pragma unroll
+        for (int i = 0; i < C::B_LOADS; i++) s[st_b + i * ROWS_STEP * C::CPR] = b_reg[i];
+    };
+
+    acc_t acc[C::TM][C::TN];
+#pragma unroll
+    for (int i = 0; i < C::TM; i++)
+#pragma unroll
+        for (int j = 0; j < C::TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+    // ---- LDS -> MFMA operand addressing -----------------------------------------------------
+    const int l32 = lane & 31, khalf = lane >> 5;  // row within the 32-row tile, K half of the lane
+    const int a_row0 = wm * C::WTM + l32, b_row0 = wn * C::WTN + l32;
+
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < ktiles; kt++) {
+        const bool more = kt + 1 < ktiles;
+        if (more) load_tile(kt + 1);
+        const uint4* sA = lds + (kt & 1) * C::STAGE_CHUNKS;
+        const uint4* sB = sA + C::BM * C::CPR;
+#pragma unroll
+        for (int ks = 0; ks < C::KSUB; ks++) {
+            if constexpr (C::FP8) {
+                v8i af[C::TM], bf[C::TN];
+                const int c0 = ks * 4 + khalf * 2;
+#pragma unroll
+                for (int i = 0; i < C::TM; i++) {
+                    const int row = a_row0 + i * 32;
+                    const uint4 lo = sA[lds_chunk<C::CPR>(row, c0)], hi = sA[lds_chunk<C::CPR>(row, c0 + 1)];
+                    af[i] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+                }
+#pragma unroll
+                for (int j = 0; j < C::TN; j++) {
+                    const int row = b_row0 + j * 32;
+                    const uint4 lo = sB[lds_chunk<C::CPR>(row, c0)], hi = sB[lds_chunk<C::CPR>(row, c0 + 1)];
+                    bf[j] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+                }
+#pragma unroll
+                for (int i = 0; i < C::TM; i++)
+#pragma unroll
+                    for (int j = 0; j < C::TN; j++)
+                        acc[i][j] = (acc_t)__builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            af[i], bf[j], (v16f)acc[i][j], C::AFMT, 0, 0, 0, 0, 0);
+            } else {
+                v4i af[C::TM], bf[C::TN];
+                const int c0 = ks * 2 + khalf;
+#pragma unroll
+                for (int i = 0; i < C::TM; i++) {
+                    const uint4 v = sA[lds_chunk<C::CPR>(a_row0 + i * 32, c0)];
+                    af[i] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                }
+#pragma unroll
+                for (int j = 0; j < C::TN; j++) {
+                    const uint4 v = sB[lds_chunk<C::CPR>(b_row0 + j * 32, c0)];
+                    bf[j] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+                }
+#pragma unroll
+                for (int i = 0; i < C::TM; i++)
+#pragma unroll
+                    for (int j = 0; j < C::TN; j++)
+                        acc[i][j] = (acc_t)__builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], (v16i)acc[i][j], 0, 0, 0);
+            }
+        }
+        if (more) store_tile((kt + 1) & 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds column n = l32, rows 8*(r/4) + 4*khalf + r%4 of each tile -----
+    const bool split = gridDim.y > 1;
+    const float alpha = ep.alpha * (ep.alpha_dev ? *ep.alpha_dev : 1.0f);
+#pragma unroll
+    for (int j = 0; j < C::TN; j++) {
+        const int n = n0 + wn * C::WTN + j * 32 + l32;
+        if (n >= N) continue;
+        float sw = 1.f, bb = 0.f;
+        if (!split) {
+            if (ep.w_scale) sw = ep.w_scale[n];
+            if (ep.bias) bb = ep.beta * load_as_f32(ep.bias, ep.bias_dtype, n);
+        }
+#pragma unroll
+        for (int i = 0; i < C::TM; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + wm * C::WTM + i * 32 + 8 * (r / 4) + 4 * khalf + (r % 4);
+                if (m >= M) continue;
+                if (split) {
+                    reinterpret_cast<uint32_t*>(partials)[((int64_t)blockIdx.y * M + m) * N + n] =
+                        __builtin_bit_cast(uint32_t, acc[i][j][r]);
+                } else {
+                    if (acc_dump)
+                        reinterpret_cast<uint32_t*>(acc_dump)[(int64_t)m * N + n] = __builtin_bit_cast(uint32_t, acc[i][j][r]);
+                    const float sa = ep.a_scale ? ep.a_scale[m] : 1.f;
+                    const float v = epi_value((float)acc[i][j][r], sa, sw, alpha, bb);
+                    reinterpret_cast<uint16_t*>(out)[(int64_t)m * ldo + n] = to_out(v, ep.out_dtype);
+                }
+            }
+        }
+    }
+}
+
+// Split-K second stage: sum the partial accumulators in split order, then the epilogue.
+template <bool FP8>
+__global__ __launch_bounds__(256) void splitk_epilogue_kernel(const void* __restrict__ partials, int splits,
+                                                              int M, int N, Epilogue ep, void* __restrict__ out,
+                                                              int64_t ldo, void* __restrict__ acc_dump) {
+    const int64_t total = (int64_t)M * N;
+    const float alpha = ep.alpha * (ep.alpha_dev ? *ep.alpha_dev : 1.0f);
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int m = (int)(idx / N), n = (int)(idx - (int64_t)m * N);
+        float accf;
+        if (FP8) {
+            float s = 0.f;
+            for (int i = 0; i < splits; i++) s += reinterpret_cast<const float*>(partials)[i * total + idx];
+            if (acc_dump) reinterpret_cast<float*>(acc_dump)[idx] = s;
+            accf = s;
+        } else {
+            int s = 0;
+            for (int i = 0; i < splits; i++) s += reinterpret_cast<const int*>(partials)[i * total + idx];
+            if (acc_dump) reinterpret_cast<int*>(acc_dump)[idx] = s;
+            accf = (float)s;
+        }
+        const float sa = ep.a_scale ? ep.a_scale[m] : 1.f, sw = ep.w_scale ? ep.w_scale[n] : 1.f;
+        const float bb = ep.bias ? ep.beta * load_as_f32(ep.bias, ep.bias_dtype, n) : 0.f;
+        reinterpret_cast<uint16_t*>(out)[(int64_t)m * ldo + n] = to_out(epi_value(accf, sa, sw, alpha, bb), ep.out_dtype);
+    }
+}
+
+// ---- host side ------------------------------------------------------------------------------
+struct Plan {
+    int cfg;     // index into the config table
+    int splits;  // K splits (1 = fused epilogue)
+    int k_per_split;
+};
+
+constexpr int kNumCu = 256;
+inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+struct TileShape { int bm, bn, bk; };
+constexpr TileShape kShapes[] = {
+    {256, 256, 64},   // 0: 4 waves x (128x128)
+    {256, 256, 64},   // 1: 8 waves x (128x64)
+    {256, 128, 64},   // 2: 4 waves x (128x64)
+    {128, 128, 64},   // 3: 4 waves x (64x64)
+    {64, 128, 128},   // 4: 4 waves x (32x64)
+    {32, 128, 128},   // 5: 4 waves x (32x32), decode
+};
+constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
+
+// Tuning/diagnostic knob (llmq_gemm_force_plan): forces a tile configuration and K split.
+int g_force_cfg = -1, g_force_splits = 1;
+bool plan_override(int& cfg, int& splits) {
+    if (g_force_cfg < 0) return false;
+    cfg = g_force_cfg;
+    splits = g_force_splits;
+    return true;
+}
+
+// Pick the tile shape and K split with the smallest modelled time:
+// waves of blocks over the CUs x per-block MFMA time, with a floor from the bytes each block streams.
+Plan make_plan(int64_t M, int64_t N, int64_t K) {
+    int ocfg, osp;
+    if (plan_override(ocfg, osp)) {
+        const TileShape s = kShapes[ocfg < kNumShapes ? ocfg : kNumShapes - 1];
+        const int kps = cdiv(cdiv(K, osp), s.bk) * s.bk;
+        return Plan{ocfg < kNumShapes ? ocfg : kNumShapes - 1, cdiv(K, kps), kps};
+    }
+    Plan best{0, 1, (int)K};
+    double best_t = 1e300;
+    for (int c = 0; c < kNumShapes; c++) {
+        const TileShape s = kShapes[c];
+        if (c == 0) continue;                                             // kept for tuning runs only
+        if (s.bm > 32 && M <= s.bm / 2 && c != kNumShapes - 1) continue;  // mostly padding
+        const int64_t tiles = (int64_t)cdiv(M, s.bm) * cdiv(N, s.bn);
+        const int max_split = (int)std::min<int64_t>(16, K / (4 * s.bk) > 0 ? K / (4 * s.bk) : 1);
+        for (int sp = 1; sp <= max_split; sp *= 2) {
+            const int kps = cdiv(cdiv(K, sp), s.bk) * s.bk;
+            const int eff_sp = cdiv(K, kps);
+            const int64_t blocks = tiles * eff_sp;
+            const int per_cu = (s.bm * s.bn >= 256 * 128) ? 1 : 2;  // resident blocks per CU
+            const double rounds = (double)cdiv(blocks, (int64_t)kNumCu * per_cu);
+            // per block: MFMA cycles at 4 SIMDs (2048 op/clk each) vs bytes streamed at ~20 B/clk/CU
+            const double mfma = 2.0 * s.bm * s.bn * kps / (4 * 2048.0) * per_cu;
+            const double bytes = (double)(s.bm + s.bn) * kps / 24.0 * per_cu;
+            double t = rounds * (std::max(mfma, bytes) + 2000.0);
+            if (eff_sp > 1) t += 6000.0 + (double)M * N * eff_sp * 4.0 / (kNumCu * 16.0);
+            if (t < best_t) { best_t = t; best = Plan{c, eff_sp, kps}; }
+        }
+    }
+    return best;
+}
+
+template <class C>
+int launch_cfg(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, int M, int N, int K, const Plan& p,
+               const Epilogue& ep, void* out, int64_t ldo, void* acc_dump, void* ws, hipStream_t st) {
+    if (C::LDS_BYTES > 65536u &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<C>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES) != hipSuccess)
+        return LLMQ_ERR_LAUNCH;
+    const int tiles = cdiv(M, C::BM) * cdiv(N, C::BN);
+    hipLaunchKernelGGL((gemm_tile_kernel<C>), dim3(tiles, p.splits), dim3(C::NT), C::LDS_BYTES, st, A, lda, B, ldb,
+                       M, N, K, p.k_per_split, ep, out, ldo, acc_dump, ws);
+    return launch_status();
+}
+
+template <bool FP8, int AFMT>
+int launch_gemm(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, int M, int N, int K, const Plan& p,
+                const Epilogue& ep, void* out, int64_t ldo, void* acc_dump, void* ws, hipStream_t st) {
+    int rc;
+    switch (p.cfg) {
+        case 0: rc = launch_cfg<GemmCfg<256, 256, 64, 2, 2, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
+        case 1: rc = launch_cfg<GemmCfg<256, 256, 64, 2, 4, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
+        case 2: rc = launch_cfg<GemmCfg<256, 128, 64, 2, 2, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
+        case 3: rc = launch_cfg<GemmCfg<128, 128, 64, 2, 2, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
+        case 4: rc = launch_cfg<GemmCfg<64, 128, 128, 2, 2, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
+        default: rc = launch_cfg<GemmCfg<32, 128, 128, 1, 4, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
+    }
+    if (rc != LLMQ_OK || p.splits == 1) return rc;
+    const int64_t total = (int64_t)M * N;
+    const int blocks = (int)std::min<int64_t>((total + 255) / 256, 4096);
+    hipLaunchKernelGGL((splitk_epilogue_kernel<FP8>), dim3(blocks), dim3(256), 0, st, ws, p.splits, M, N, ep, out, ldo,
+                       acc_dump);
+    return launch_status();
+}
+
+int gemm_entry(bool fp8, int a_format, const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb,
+               const float* a_scale, const float* w_scale, float alpha, const float* alpha_dev, const void* bias,
+               int bias_dtype, float beta, void* out, int out_dtype, int64_t ldo, int64_t M, int64_t N, int64_t K,
+               void* acc_dump, void* ws, size_t ws_bytes, hipStream_t st) {
+    if (M < 0 || N < 0 || K < 0) return LLMQ_ERR_SHAPE;
+    if (M == 0 || N == 0) return LLMQ_OK;
+    if (!A || !B || !out) return LLMQ_ERR_NULL;
+    if (K == 0 || (K & 15) || (lda & 15) || (ldb & 15) || lda < K || ldb < K || ldo < N) return LLMQ_ERR_SHAPE;
+    if (M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL || lda >= (1 << 22) || ldb >= (1 << 22)) return LLMQ_ERR_SHAPE;
+    if (out_dtype != LLMQ_BF16 && out_dtype != LLMQ_F16) return LLMQ_ERR_DTYPE;
+    if (bias && bias_dtype != LLMQ_BF16 && bias_dtype != LLMQ_F16 && bias_dtype != LLMQ_F32) return LLMQ_ERR_DTYPE;
+    if (fp8 && a_format != LLMQ_E4M3 && a_format != LLMQ_E5M2) return LLMQ_ERR_DTYPE;
+    if (!aligned16(A) || !aligned16(B)) return LLMQ_ERR_ALIGN;
+    const Plan p = make_plan(M, N, K);
+    if (p.splits > 1) {
+        if (!ws || ws_bytes < (size_t)p.splits * M * N * 4) return LLMQ_ERR_WORKSPACE;
+    }
+    Epilogue ep{a_scale, w_scale, alpha_dev, bias, alpha, beta, bias_dtype, out_dtype};
+    if (!fp8) return launch_gemm<false, 0>(A, lda, B, ldb, (int)M, (int)N, (int)K, p, ep, out, ldo, acc_dump, ws, st);
+    if (a_format == LLMQ_E4M3)
+        return launch_gemm<true, 0>(A, lda, B, ldb, (int)M, (int)N, (int)K, p, ep, out, ldo, acc_dump, ws, st);
+    return launch_gemm<true, 1>(A, lda, B, ldb, (int)M, (int)N, (int)K, p, ep, out, ldo, acc_dump, ws, st);
+}
+
+}  // namespace
+}  // namespace llmq
+
+using namespace llmq;
+
+extern "C" int llmq_gemm_force_plan(int cfg, int splits) {
+    if (cfg >= kNumShapes || splits < 1 || splits > 64) return LLMQ_ERR_SHAPE;
+    g_force_cfg = cfg;
+    g_force_splits = splits;
+    return LLMQ_OK;
+}
+
+extern "C" int llmq_gemm_num_configs(void) { return kNumShapes; }
+
+extern "C" size_t llmq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const Plan p = make_plan(M, N, K);
+    return p.splits > 1 ? (size_t)p.splits * M * N * 4 : 0;
+}
+
+extern "C" int llmq_gemm_w8a8(const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb, const float* a_scale,
+                              const float* w_scale, float alpha, const float* alpha_dev, const void* bias,
+                              int bias_dtype, float beta, void* out, int out_dtype, int64_t ldo, int64_t M, int64_t N,
+                              int64_t K, int32_t* acc_dump, void* workspace, size_t workspace_bytes,
+                              llmq_stream_t stream) {
+    return gemm_entry(false, 0, (const uint8_t*)A, lda, (const uint8_t*)B, ldb, a_scale, w_scale, alpha, alpha_dev,
+                      bias, bias_dtype, beta, out, out_dtype, ldo, M, N, K, acc_dump, workspace, workspace_bytes,
+                      (hipStream_t)stream);
+}
+
+extern "C" int llmq_gemm_fp8(const uint8_t* A, int a_format, int64_t lda, const uint8_t* B, int64_t ldb,
+                             const float* a_scale, const float* w_scale, float alpha, const float* alpha_dev,
+                             const void* bias, int bias_dtype, float beta, void* out, int out_dtype, int64_t ldo,
+                             int64_t M, int64_t N, int64_t K, float* acc_dump, void* workspace,
+                             size_t workspace_bytes, llmq_stream_t stream) {
+    return gemm_entry(true, a_format, A, lda, B, ldb, a_scale, w_scale, alpha, alpha_dev, bias, bias_dtype, beta, out,
+                      out_dtype, ldo, M, N, K, acc_dump, workspace, workspace_bytes, (hipStream_t)stream);
+}

@@ -1,0 +1,58 @@
+// Shared device/host helpers for the gfx950 kernels of libllmq_gfx950.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "llmq.h"
+
+namespace llmq {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// ---- 16-bit float storage types, handled as raw bits + fp32 math -------------------------
+template <int DT> struct Lo;
+template <> struct Lo<LLMQ_BF16> {
+    static __device__ __forceinline__ float to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+    static __device__ __forceinline__ uint16_t from_f32(float f) {  // round to nearest even
+        return __builtin_bit_cast(uint16_t, (__bf16)f);
+    }
+    static __device__ __forceinline__ float round(float f) { return to_f32(from_f32(f)); }
+};
+template <> struct Lo<LLMQ_F16> {
+    static __device__ __forceinline__ float to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+    static __device__ __forceinline__ uint16_t from_f32(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+    static __device__ __forceinline__ float round(float f) { return to_f32(from_f32(f)); }
+};
+
+__device__ __forceinline__ float load_as_f32(const void* p, int dtype, int64_t i) {
+    if (dtype == LLMQ_F32) return ((const float*)p)[i];
+    uint16_t h = ((const uint16_t*)p)[i];
+    return dtype == LLMQ_BF16 ? Lo<LLMQ_BF16>::to_f32(h) : Lo<LLMQ_F16>::to_f32(h);
+}
+
+// ---- wavefront / block reductions ---------------------------------------------------------
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+// max over a block of NW wavefronts; every thread gets the result.  `smem` holds NW floats.
+template <int NW>
+__device__ __forceinline__ float block_max(float v, float* smem) {
+    v = wave_max(v);
+    const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+    __syncthreads();  // smem may still be read from a previous call
+    if (lane == 0) smem[w] = v;
+    __syncthreads();
+    float r = smem[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) r = fmaxf(r, smem[i]);
+    return r;
+}
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? LLMQ_OK : LLMQ_ERR_LAUNCH; }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace llmq

@@ -1,0 +1,301 @@
+// Activation quantizers (int8 SmoothQuant and OCP e4m3fn FP8), one fused HIP kernel each.
+//
+// The reference runs these as chains of eager torch ops in the activation dtype
+// (nn_models/modules/linear/linear_sq.py:44-65, nn_models/modules/linear/linear_fp8.py:11-63):
+//   scale = round_dt( max(absmax, round_dt(floor)) / qmax )
+//   q     = narrow( clamp( round_dt( x / scale ) ) )
+// The kernels reproduce exactly that sequence of roundings.  They are HBM-bound:
+// 2 bytes read + 1 byte written per element, one row per 256-thread block, the row held in
+// registers between the absmax pass and the quantize pass so x is read from HBM once.
+#include "llmq_common.h"
+
+namespace llmq {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kNW = kThreads / kWave;
+constexpr int kMaxPartials = 1024;  // per-tensor absmax partials (one per stage-1 block)
+
+enum { MODE_I8 = 0, MODE_F8 = 1 };
+enum { SCALE_ROW = 0, SCALE_TENSOR = 1, SCALE_STATIC = 2 };
+
+template <int MODE> struct QP;
+template <> struct QP<MODE_I8> { static constexpr float floor_ = 1e-5f, qmax = 127.f, lo = -128.f, hi = 127.f; };
+template <> struct QP<MODE_F8> { static constexpr float floor_ = 1e-12f, qmax = 448.f, lo = -448.f, hi = 448.f; };
+
+template <int DT, int MODE>
+__device__ __forceinline__ float scale_from_amax(float amax) {
+    const float fl = Lo<DT>::round(QP<MODE>::floor_);  // the clamp bound lives in the activation dtype
+    return Lo<DT>::round(fmaxf(amax, fl) / QP<MODE>::qmax);
+}
+
+__device__ __forceinline__ float absmax8(uint4 r, int dt_is_bf16) {
+    // |x| of 8 packed 16-bit floats: clear the sign bits, compare as fp32
+    const uint32_t w[4] = {r.x & 0x7fff7fffu, r.y & 0x7fff7fffu, r.z & 0x7fff7fffu, r.w & 0x7fff7fffu};
+    float m = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float a, b;
+        if (dt_is_bf16) {
+            a = __uint_as_float(w[i] << 16);
+            b = __uint_as_float(w[i] & 0xffff0000u);
+        } else {
+            a = Lo<LLMQ_F16>::to_f32((uint16_t)(w[i] & 0xffffu));
+            b = Lo<LLMQ_F16>::to_f32((uint16_t)(w[i] >> 16));
+        }
+        m = fmaxf(m, fmaxf(a, b));
+    }
+    return m;
+}
+
+// Quotient rounded to the activation dtype.  bf16: x * (1/s) rounds to the same bf16 value
+// as the exact quotient for every pair of bf16 operands (the exact quotient of two 8-bit
+// significands is never closer than 2^-17 relative to a bf16 rounding boundary), so one
+// multiply replaces the division.  fp16 significands are too long for that: true division.
+// Q_DT: scale is itself a value of the activation dtype (dynamic quantizers).
+// Q_DIV_DT: arbitrary fp32 scale, quotient rounded to the activation dtype (tensor / Python float).
+// Q_DIV_F32: arbitrary fp32 scale, quotient kept in fp32 (tensor / fp32 tensor promotes).
+enum { Q_DT = 0, Q_DIV_DT = 1, Q_DIV_F32 = 2 };
+template <int DT, int QUOT>
+__device__ __forceinline__ float quotient(float x, float s, float inv_s) {
+    if (QUOT == Q_DIV_F32) return x / s;
+    if (QUOT == Q_DIV_DT || DT == LLMQ_F16) return Lo<DT>::round(x / s);
+    return Lo<DT>::round(x * inv_s);
+}
+
+template <int DT, int MODE, int QUOT>
+__device__ __forceinline__ uint2 quant8(uint4 raw, float s, float inv_s) {
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        f[2 * i] = Lo<DT>::to_f32((uint16_t)(w[i] & 0xffffu));
+        f[2 * i + 1] = Lo<DT>::to_f32((uint16_t)(w[i] >> 16));
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        float q = quotient<DT, QUOT>(f[i], s, inv_s);
+        const float c = __builtin_amdgcn_fmed3f(q, QP<MODE>::lo, QP<MODE>::hi);
+        f[i] = (q != q) ? q : c;  // clamp keeps NaN, as torch.clamp does
+    }
+    uint32_t out[2];
+    if (MODE == MODE_I8) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            uint32_t b[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                // adding 1.5*2^23 rounds to the nearest integer, ties to even, and leaves the
+                // two's-complement value in the low mantissa bits
+                const float v = f[4 * h + i];
+                b[i] = (v != v) ? 0u : (__float_as_uint(v + 12582912.0f) & 0xffu);
+            }
+            out[h] = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+        }
+    } else {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            int p = 0;
+            p = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * h + 0], f[4 * h + 1], p, false);
+            p = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * h + 2], f[4 * h + 3], p, true);
+            out[h] = (uint32_t)p;
+        }
+    }
+    return make_uint2(out[0], out[1]);
+}
+
+// One block per row.  NC > 0: the row's 16-byte chunks (8 elements) are kept in NC
+// registers per thread between the two passes; NC == 0: rows of any length, second pass
+// re-reads x (served by L2).
+template <int DT, int MODE, int SCALE, int NC>
+__global__ __launch_bounds__(kThreads) void quant_rows_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, int64_t K, uint8_t* __restrict__ q,
+    void* __restrict__ scale_out, int scale_dtype, const float* __restrict__ aux, int n_aux,
+    int static_f32) {
+    __shared__ float smem[kNW];
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int nchunk = (int)(K >> 3);
+    const uint4* xr = reinterpret_cast<const uint4*>(x + row * ldx);
+    uint2* qr = reinterpret_cast<uint2*>(q + row * K);
+
+    uint4 cache[NC > 0 ? NC : 1];
+    float s;
+    if (SCALE == SCALE_ROW) {
+        float amax = 0.f;
+        if (NC > 0) {
+#pragma unroll
+            for (int c = 0; c < NC; c++) {
+                const int i = tid + c * kThreads;
+                cache[c] = (i < nchunk) ? xr[i] : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int c = 0; c < NC; c++) amax = fmaxf(amax, absmax8(cache[c], DT == LLMQ_BF16));
+        } else {
+            for (int i = tid; i < nchunk; i += kThreads) amax = fmaxf(amax, absmax8(xr[i], DT == LLMQ_BF16));
+        }
+        amax = block_max<kNW>(amax, smem);
+        s = scale_from_amax<DT, MODE>(amax);
+    } else if (SCALE == SCALE_TENSOR) {
+        float amax = 0.f;
+        for (int i = tid; i < n_aux; i += kThreads) amax = fmaxf(amax, aux[i]);
+        amax = block_max<kNW>(amax, smem);
+        s = scale_from_amax<DT, MODE>(amax);
+    } else {
+        s = aux[0];
+    }
+    if (SCALE != SCALE_STATIC && tid == 0 && (SCALE == SCALE_ROW || row == 0)) {
+        const int64_t o = SCALE == SCALE_ROW ? row : 0;
+        if (scale_dtype == LLMQ_F32) ((float*)scale_out)[o] = s;
+        else ((uint16_t*)scale_out)[o] = Lo<DT>::from_f32(s);
+    }
+    const float inv_s = 1.0f / s;
+    constexpr bool F32Q = (SCALE == SCALE_STATIC);
+    if (SCALE == SCALE_ROW && NC > 0) {
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+            const int i = tid + c * kThreads;
+            if (i < nchunk) qr[i] = quant8<DT, MODE, Q_DT>(cache[c], s, inv_s);
+        }
+    } else if (F32Q) {
+        if (static_f32) {
+            for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, MODE, Q_DIV_F32>(xr[i], s, inv_s);
+        } else {
+            for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, MODE, Q_DIV_DT>(xr[i], s, inv_s);
+        }
+    } else {
+        for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, MODE, Q_DT>(xr[i], s, inv_s);
+    }
+}
+
+// Stage 1 of the per-tensor quantizers: grid-stride absmax, one partial per block.
+template <int DT>
+__global__ __launch_bounds__(kThreads) void absmax_partials_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, int64_t M, int64_t K, float* __restrict__ partials) {
+    __shared__ float smem[kNW];
+    const int64_t cpr = K >> 3, total = M * cpr;
+    float amax = 0.f;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kThreads) {
+        const int64_t r = i / cpr, c = i - r * cpr;
+        amax = fmaxf(amax, absmax8(reinterpret_cast<const uint4*>(x + r * ldx)[c], DT == LLMQ_BF16));
+    }
+    amax = block_max<kNW>(amax, smem);
+    if (threadIdx.x == 0) partials[blockIdx.x] = amax;
+}
+
+int check_common(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, const void* q) {
+    if (!x || !q) return (M == 0 || K == 0) ? LLMQ_OK : LLMQ_ERR_NULL;
+    if (x_dtype != LLMQ_BF16 && x_dtype != LLMQ_F16) return LLMQ_ERR_DTYPE;
+    if (M < 0 || K < 0 || ldx < K || (K & 7) || (ldx & 7) || M > 0x7fffffffLL) return LLMQ_ERR_SHAPE;
+    if (!aligned16(x) || (reinterpret_cast<uintptr_t>(q) & 7u)) return LLMQ_ERR_ALIGN;
+    return LLMQ_OK;
+}
+
+template <int DT, int MODE, int SCALE>
+int launch_rows(const void* x, int64_t M, int64_t K, int64_t ldx, void* q, void* scale, int scale_dtype,
+                const float* aux, int n_aux, int static_f32, hipStream_t st) {
+    const dim3 grid((unsigned)M), block(kThreads);
+    const uint16_t* xp = (const uint16_t*)x;
+    uint8_t* qp = (uint8_t*)q;
+    const int64_t per_thread = ((K >> 3) + kThreads - 1) / kThreads;
+#define LLMQ_LAUNCH_NC(NC) \
+    hipLaunchKernelGGL((quant_rows_kernel<DT, MODE, SCALE, NC>), grid, block, 0, st, xp, ldx, K, qp, scale, scale_dtype, aux, n_aux, static_f32)
+    if (SCALE != SCALE_ROW) LLMQ_LAUNCH_NC(0);
+    else if (per_thread <= 1) LLMQ_LAUNCH_NC(1);
+    else if (per_thread <= 2) LLMQ_LAUNCH_NC(2);
+    else if (per_thread <= 4) LLMQ_LAUNCH_NC(4);
+    else if (per_thread <= 10) LLMQ_LAUNCH_NC(10);
+    else LLMQ_LAUNCH_NC(0);
+#undef LLMQ_LAUNCH_NC
+    return launch_status();
+}
+
+template <int MODE, int SCALE>
+int dispatch_rows(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, void* q, void* scale,
+                  int scale_dtype, const float* aux, int n_aux, int static_f32, hipStream_t st) {
+    if (x_dtype == LLMQ_BF16)
+        return launch_rows<LLMQ_BF16, MODE, SCALE>(x, M, K, ldx, q, scale, scale_dtype, aux, n_aux, static_f32, st);
+    return launch_rows<LLMQ_F16, MODE, SCALE>(x, M, K, ldx, q, scale, scale_dtype, aux, n_aux, static_f32, st);
+}
+
+template <int MODE>
+int per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, void* q, void* scale,
+               int scale_dtype, void* ws, size_t ws_bytes, hipStream_t st) {
+    if (!ws || ws_bytes < kMaxPartials * sizeof(float)) return LLMQ_ERR_WORKSPACE;
+    const int64_t total = M * (K >> 3);
+    int nblk = (int)((total + kThreads * 4 - 1) / (kThreads * 4));
+    nblk = nblk < 1 ? 1 : (nblk > kMaxPartials ? kMaxPartials : nblk);
+    float* partials = (float*)ws;
+    if (x_dtype == LLMQ_BF16)
+        hipLaunchKernelGGL((absmax_partials_kernel<LLMQ_BF16>), dim3(nblk), dim3(kThreads), 0, st,
+                           (const uint16_t*)x, ldx, M, K, partials);
+    else
+        hipLaunchKernelGGL((absmax_partials_kernel<LLMQ_F16>), dim3(nblk), dim3(kThreads), 0, st,
+                           (const uint16_t*)x, ldx, M, K, partials);
+    if (launch_status() != LLMQ_OK) return LLMQ_ERR_LAUNCH;
+    return dispatch_rows<MODE, SCALE_TENSOR>(x, x_dtype, M, K, ldx, q, scale, scale_dtype, partials, nblk, 0, st);
+}
+
+}  // namespace
+}  // namespace llmq
+
+using namespace llmq;
+
+extern "C" size_t llmq_quant_workspace_bytes(void) { return kMaxPartials * sizeof(float); }
+
+extern "C" int llmq_quant_i8_per_token(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                       int8_t* q, void* scale, int scale_dtype, llmq_stream_t stream) {
+    int rc = check_common(x, x_dtype, M, K, ldx, q);
+    if (rc != LLMQ_OK) return rc;
+    if (M == 0) return LLMQ_OK;
+    if (!scale) return LLMQ_ERR_NULL;
+    if (scale_dtype != x_dtype && scale_dtype != LLMQ_F32) return LLMQ_ERR_DTYPE;
+    if (K == 0) return LLMQ_ERR_SHAPE;
+    return dispatch_rows<MODE_I8, SCALE_ROW>(x, x_dtype, M, K, ldx, q, scale, scale_dtype, nullptr, 0, 0,
+                                             (hipStream_t)stream);
+}
+
+extern "C" int llmq_quant_i8_per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                        int8_t* q, void* scale, int scale_dtype, void* workspace,
+                                        size_t workspace_bytes, llmq_stream_t stream) {
+    int rc = check_common(x, x_dtype, M, K, ldx, q);
+    if (rc != LLMQ_OK) return rc;
+    if (!scale) return LLMQ_ERR_NULL;
+    if (scale_dtype != x_dtype && scale_dtype != LLMQ_F32) return LLMQ_ERR_DTYPE;
+    if (M == 0 || K == 0) return LLMQ_ERR_SHAPE;
+    return per_tensor<MODE_I8>(x, x_dtype, M, K, ldx, q, scale, scale_dtype, workspace, workspace_bytes,
+                               (hipStream_t)stream);
+}
+
+extern "C" int llmq_quant_fp8_per_token(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                        uint8_t* q, float* scale, llmq_stream_t stream) {
+    int rc = check_common(x, x_dtype, M, K, ldx, q);
+    if (rc != LLMQ_OK) return rc;
+    if (M == 0) return LLMQ_OK;
+    if (!scale) return LLMQ_ERR_NULL;
+    if (K == 0) return LLMQ_ERR_SHAPE;
+    return dispatch_rows<MODE_F8, SCALE_ROW>(x, x_dtype, M, K, ldx, q, scale, LLMQ_F32, nullptr, 0, 0,
+                                             (hipStream_t)stream);
+}
+
+extern "C" int llmq_quant_fp8_per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                         uint8_t* q, float* scale, void* workspace, size_t workspace_bytes,
+                                         llmq_stream_t stream) {
+    int rc = check_common(x, x_dtype, M, K, ldx, q);
+    if (rc != LLMQ_OK) return rc;
+    if (!scale) return LLMQ_ERR_NULL;
+    if (M == 0 || K == 0) return LLMQ_ERR_SHAPE;
+    return per_tensor<MODE_F8>(x, x_dtype, M, K, ldx, q, scale, LLMQ_F32, workspace, workspace_bytes,
+                               (hipStream_t)stream);
+}
+
+extern "C" int llmq_quant_fp8_static(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                     uint8_t* q, const float* scale, int scale_is_f32_tensor,
+                                     llmq_stream_t stream) {
+    int rc = check_common(x, x_dtype, M, K, ldx, q);
+    if (rc != LLMQ_OK) return rc;
+    if (M == 0 || K == 0) return LLMQ_OK;
+    if (!scale) return LLMQ_ERR_NULL;
+    return dispatch_rows<MODE_F8, SCALE_STATIC>(x, x_dtype, M, K, ldx, q, nullptr, LLMQ_F32, scale, 1,
+                                                scale_is_f32_tensor ? 1 : 0, (hipStream_t)stream);
+}
