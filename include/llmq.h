@@ -4,8 +4,9 @@
  * Conventions
  *  - Every pointer is a DEVICE pointer unless its comment says "host".
  *  - The caller owns every buffer (inputs, outputs, workspaces); the library allocates
- *    nothing, keeps no state between calls, never synchronises with the host and launches
- *    on the stream it is given (0 = the null stream).  Calls are asynchronous.
+ *    nothing, keeps no state between calls (llmq_gemm_force_plan, a tuning hook, is the one
+ *    exception), never synchronises with the host and launches on the stream it is given
+ *    (0 = the null stream).  Calls are asynchronous.
  *  - Matrices are row-major; `ld*` is the row stride in ELEMENTS.
  *  - Return value: LLMQ_OK (0) or a negative llmq_status; llmq_status_string() names it.
  *  - Paths below are relative to the reference's runtime/ directory.
@@ -68,8 +69,8 @@ int llmq_quant_fp8_per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, 
                               void* workspace, size_t workspace_bytes, llmq_stream_t stream);
 
 /* Replaces static_per_tensor_quantize, linear_fp8.py:34-37.  scale: fp32 device scalar; the
- * quotient is formed in fp32 (tensor / fp32 tensor promotes) when scale_is_f32_tensor != 0,
- * else the scalar is first rounded to x_dtype and the quotient rounded to x_dtype. */
+ * quotient x / scale is kept in fp32 (torch: tensor / fp32 tensor promotes) when
+ * scale_is_f32_tensor != 0, else it is rounded to x_dtype (torch: tensor / Python float). */
 int llmq_quant_fp8_static(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
                           uint8_t* q, const float* scale, int scale_is_f32_tensor,
                           llmq_stream_t stream);

@@ -1,0 +1,88 @@
+"""GPU parity: AWQ W4A16 kernels vs the CPU oracle.
+
+Dequantized weights: bit-exact.  GEMM: max |y - y_ref| / max |y_ref| <= 1e-2 against
+dequantize-then-matmul with fp32 accumulation (the reference's own fallback math; its Triton kernel
+accumulates in fp16 with atomics and is not a bit-level oracle).
+"""
+import pytest
+import torch
+
+from oracle import ref_math as R
+
+pytestmark = pytest.mark.gpu
+REL_TOL = 1e-2
+
+
+def rel_err(y, ref):
+    y, ref = y.float().cpu(), ref.float()
+    return ((y - ref).abs().max() / ref.abs().max().clamp(min=1e-30)).item()
+
+
+@pytest.mark.parametrize("K,N,G", [(3584, 4608, 128), (896, 4864, 128), (256, 264, 64), (128, 8, 32), (512, 1000, 512)])
+def test_dequant_bit_exact(cuda, K, N, G):
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_dequantize_triton
+    qw, qz, s = W.awq_weights(N, K, K + N, group=G)
+    ref = R.awq_dequantize(qw, qz, s, G)
+    out = awq_dequantize_triton(qw.to(cuda), s.to(cuda), qz.to(cuda))
+    assert out.dtype == torch.float16 and out.shape == (K, N)
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+def test_dequant_all_nibble_values(cuda):
+    """Every (q, z) pair in every nibble slot, with scales that exercise fp16 rounding and subnormals."""
+    from llmqrt_amd.awq_kernels import awq_dequantize_triton
+    K, N = 256, 16
+    g = torch.Generator().manual_seed(1)
+    q = torch.arange(K, dtype=torch.int32).view(K, 1).expand(K, N) % 16
+    q = (q + torch.arange(N, dtype=torch.int32).view(1, N)) % 16
+    z = torch.randint(0, 16, (K // 32, N), generator=g, dtype=torch.int32)
+    s = torch.rand(K // 32, N, generator=g).half() * 0.01
+    s[0, :4] = torch.tensor([6.0e-8, 1.0e-5, 0.333, 1000.0]).half()
+    qw, qz = R.awq_pack(q), R.awq_pack(z)
+    ref = R.awq_dequantize(qw, qz, s, 32)
+    out = awq_dequantize_triton(qw.to(cuda), s.to(cuda), qz.to(cuda))
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("M", [1, 4, 16, 64])
+@pytest.mark.parametrize("K,N", [(3584, 4608), (896, 4864)])
+def test_gemm_decode_shapes(cuda, M, K, N):
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    qw, qz, s = W.awq_weights(N, K, 3000 + M, group=128)
+    x = W.activations(M, K, 3100 + M, dtype=torch.float16, outliers=False)
+    ref = R.awq_gemm(x, qw, qz, s, 128)
+    out = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8)
+    assert out.dtype == torch.float16 and out.shape == (M, N)
+    assert rel_err(out, ref) <= REL_TOL
+    out2 = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8)
+    assert torch.equal(out, out2), "the kernel must be deterministic"
+
+
+@pytest.mark.parametrize("M,K,N,G", [(3, 256, 264, 64), (17, 128, 8, 32), (5, 512, 1000, 512), (65, 1024, 136, 128),
+                                     (130, 256, 2048, 128), (2, 18944, 3584, 128), (16, 3584, 37888, 128)])
+def test_gemm_ragged_and_wide(cuda, M, K, N, G):
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    qw, qz, s = W.awq_weights(N, K, 5 * M + N, group=G)
+    x = W.activations(M, K, 6 * M + K, dtype=torch.float16, outliers=False)
+    ref = R.awq_gemm(x, qw, qz, s, G)
+    out = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8)
+    assert rel_err(out, ref) <= REL_TOL
+
+
+def test_gemm_asserts_like_reference(cuda):
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    qw = torch.zeros(128, 16, dtype=torch.int32, device=cuda)
+    qz = torch.zeros(1, 16, dtype=torch.int32, device=cuda)
+    s = torch.ones(1, 128, dtype=torch.float16, device=cuda)
+    x = torch.ones(2, 128, dtype=torch.float16, device=cuda)
+    with pytest.raises(AssertionError):
+        awq_gemm_triton(x, qw, s, qz, split_k_iters=3)     # not a power of two
+    with pytest.raises(AssertionError):
+        awq_gemm_triton(x, qw, s, qz, split_k_iters=64)    # > 32
+    with pytest.raises(AssertionError):
+        awq_gemm_triton(x[:, :64], qw, s, qz, split_k_iters=8)
+    out = awq_gemm_triton(x, qw, s, qz, split_k_iters=8)    # all-zero q and z -> zeros
+    assert torch.count_nonzero(out).item() == 0

@@ -1,0 +1,132 @@
+"""GPU parity: activation quantizers vs the CPU oracle, bit-exact (integer/byte outputs and scales)."""
+import pytest
+import torch
+
+from oracle import ref_math as R
+
+pytestmark = pytest.mark.gpu
+
+
+def _acts(M, K, seed, dtype):
+    from llmqrt_amd import workloads as W
+    return W.activations(M, K, seed, dtype=dtype)
+
+
+SHAPES = [(1, 896), (16, 896), (7, 3584), (128, 3584), (33, 18944), (3, 8), (5, 24576), (2, 40960)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K", SHAPES)
+def test_int8_per_token(cuda, M, K, dtype):
+    from llmqrt_amd.quantize import quantize_activation_per_token_absmax, quantize_activation_per_token_absmax_f32
+    x = _acts(M, K, 11 * M + K, dtype)
+    x[0, : min(K, 64)] = 0  # exercise exact zeros
+    if M > 2:
+        x[2] = 0            # an all-zero row: scale = round(round(1e-5)/127)
+    q_ref, s_ref = R.quantize_activation_per_token_absmax(x)
+    q, s = quantize_activation_per_token_absmax(x.to(cuda))
+    assert q.dtype == torch.int8 and s.dtype == dtype and s.shape == (M, 1)
+    assert torch.equal(s.cpu().view(torch.int16), s_ref.view(torch.int16))
+    assert torch.equal(q.cpu(), q_ref)
+    q2, s2 = quantize_activation_per_token_absmax_f32(x.to(cuda))
+    assert torch.equal(q2.cpu(), q_ref) and torch.equal(s2.cpu(), s_ref.float())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K", SHAPES)
+def test_fp8_per_token(cuda, M, K, dtype):
+    from llmqrt_amd.quantize import per_token_quantize
+    x = _acts(M, K, 13 * M + K, dtype)
+    if M > 2 and dtype == torch.bfloat16:
+        x[2] = 0  # fp16 zero rows give scale 0 -> NaN in the reference; covered separately
+    q_ref, s_ref = R.fp8_per_token_quantize(x)
+    q, s = per_token_quantize(x.to(cuda))
+    assert q.dtype == torch.float8_e4m3fn and s.dtype == torch.float32 and s.shape == (M, 1)
+    assert torch.equal(s.cpu(), s_ref)
+    assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
+
+
+def test_fp16_zero_row_fp8_is_nan_like_reference(cuda):
+    from llmqrt_amd.quantize import per_token_quantize
+    x = torch.zeros(2, 64, dtype=torch.float16)
+    x[1] = 1.0
+    q_ref, s_ref = R.fp8_per_token_quantize(x)
+    q, s = per_token_quantize(x.to(cuda))
+    assert torch.equal(s.cpu(), s_ref)
+    assert torch.equal(q.cpu().view(torch.uint8), q_ref.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_all_16bit_patterns(cuda, dtype):
+    """Every finite 16-bit pattern as an input element, against several row maxima."""
+    from llmqrt_amd.quantize import per_token_quantize, quantize_activation_per_token_absmax
+    bits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(dtype)
+    finite = bits[torch.isfinite(bits.float())]
+    n = (finite.numel() // 8) * 8
+    rows = []
+    for amax in (0.75, 3.1415, 37.5, 1000.0, 6.1e-5, 65000.0 if dtype == torch.float16 else 3.0e38):
+        r = finite[:n].clone().float()
+        r[r.abs() > amax] = 0
+        r[0] = amax
+        rows.append(r.to(dtype))
+    x = torch.stack(rows)
+    q_ref, s_ref = R.quantize_activation_per_token_absmax(x)
+    q, s = quantize_activation_per_token_absmax(x.to(cuda))
+    assert torch.equal(s.cpu().view(torch.int16), s_ref.view(torch.int16))
+    assert torch.equal(q.cpu(), q_ref)
+    f_ref, fs_ref = R.fp8_per_token_quantize(x)
+    f, fs = per_token_quantize(x.to(cuda))
+    assert torch.equal(fs.cpu(), fs_ref)
+    assert torch.equal(f.cpu().view(torch.uint8), f_ref.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K", [(16, 896), (130, 3584), (1, 8)])
+def test_per_tensor(cuda, M, K, dtype):
+    from llmqrt_amd.quantize import per_tensor_quantize, quantize_activation_per_tensor_absmax
+    x = _acts(M, K, 17 * M + K, dtype)
+    q_ref, s_ref = R.quantize_activation_per_tensor_absmax(x)
+    q, s = quantize_activation_per_tensor_absmax(x.to(cuda))
+    assert s.dim() == 0 and s.dtype == dtype
+    assert s.cpu().view(torch.int16).item() == s_ref.view(torch.int16).item()
+    assert torch.equal(q.cpu(), q_ref)
+    f_ref, fs_ref = R.fp8_per_tensor_quantize(x)
+    f, fs = per_tensor_quantize(x.to(cuda))
+    assert fs.dim() == 0 and fs.cpu().item() == fs_ref.item()
+    assert torch.equal(f.cpu().view(torch.uint8), f_ref.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_static_fp8(cuda, dtype):
+    from llmqrt_amd.quantize import static_per_tensor_quantize
+    x = _acts(64, 896, 5, dtype)
+    for scale in (0.0123456, 0.25, 1.7):
+        st = torch.tensor([scale], dtype=torch.float32)
+        ref_t = R.fp8_static_per_tensor_quantize(x, st)          # fp32 tensor scale: fp32 quotient
+        got_t = static_per_tensor_quantize(x.to(cuda), st.to(cuda))
+        assert torch.equal(got_t.cpu().view(torch.uint8), ref_t.view(torch.uint8))
+        ref_f = R.fp8_static_per_tensor_quantize(x, scale)       # Python float: quotient in x.dtype
+        got_f = static_per_tensor_quantize(x.to(cuda), scale)
+        assert torch.equal(got_f.cpu().view(torch.uint8), ref_f.view(torch.uint8))
+
+
+def test_strided_input_and_3d(cuda):
+    from llmqrt_amd.quantize import quantize_activation_per_token_absmax
+    x = _acts(8, 1024, 3, torch.bfloat16)
+    xs = x.to(cuda)[:, :512]                                     # row stride 1024, K 512
+    q_ref, s_ref = R.quantize_activation_per_token_absmax(x[:, :512].contiguous())
+    q, s = quantize_activation_per_token_absmax(xs)
+    assert torch.equal(q.cpu(), q_ref) and torch.equal(s.cpu(), s_ref)
+    x3 = x.view(2, 4, 1024)
+    q3, s3 = quantize_activation_per_token_absmax(x3.to(cuda))
+    assert q3.shape == (2, 4, 1024) and s3.shape == (2, 4, 1)
+    assert torch.equal(q3.cpu().view(8, 1024), R.quantize_activation_per_token_absmax(x)[0])
+
+
+def test_empty_rows(cuda):
+    from llmqrt_amd.quantize import per_token_quantize, quantize_activation_per_token_absmax
+    x = torch.empty(0, 64, dtype=torch.bfloat16, device=cuda)
+    q, s = quantize_activation_per_token_absmax(x)
+    assert q.shape == (0, 64) and s.shape == (0, 1)
+    q, s = per_token_quantize(x)
+    assert q.shape == (0, 64) and s.shape == (0, 1)
