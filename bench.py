@@ -1,0 +1,377 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-details] [--no-cpu]
+
+Headline (the ONE JSON line printed last): the SmoothQuant W8A8 sweep at Qwen2-7B shapes -
+projections qkv / o / gate_up / down at M in {1, 16, 128, 2048, 8192}, each linear = per-token
+dynamic int8 quantizer kernel + int8 MFMA GEMM with the per-token x per-channel dequant epilogue.
+A "step" is one pass over those 20 linears with every input already resident in HBM; `value` is
+sum(2*M*N*K) / step time in TOPS.  The same line carries
+  roofline     - the dominant kernel (int8 MFMA GEMM at the prefill shapes M >= 2048), timed per
+                 launch with HIP events on the launch stream, against the dense int8 MFMA peak;
+  cpu_baseline - the reference's dequantize-then-matmul math (the oracle) on the host cores for a
+                 bounded sample of the same workload, which also serves as the parity check;
+  details      - per-shape figures for the W8A8 sweep, the FP8 sweep, AWQ W4A16 decode (GB/s
+                 against the HBM peak) and the decoder-layer stack.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5033.0   # dense int8 MFMA peak of MI355X, TOP/s (256 CU x 2.4 GHz x 8192 op/clk)
+PEAK_FP8_TFLOPS = 5033.0  # dense fp8 MFMA peak
+PEAK_HBM_GBS = 8000.0     # HBM3E peak, GB/s
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-details", action="store_true", help="skip the per-shape FP8 / AWQ / layer tables")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="run only the dominant kernel's launches (for rocprofv3 summaries)")
+    return ap.parse_args()
+
+
+class W8A8Linear:
+    """One W8A8 linear with preallocated buffers; launch() = quantizer + GEMM through the C ABI."""
+
+    def __init__(self, name, M, K, N, qweight, w_scale, seed, dev):
+        from llmqrt_amd import _abi, workloads as W
+        self.name, self.M, self.K, self.N = name, M, K, N
+        self.x = W.activations(M, K, seed).to(dev)
+        self.qweight, self.w_scale = qweight, w_scale
+        self.qx = torch.empty((M, K), dtype=torch.int8, device=dev)
+        self.a_scale = torch.empty((M,), dtype=torch.float32, device=dev)
+        self.out = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        L = _abi.lib()
+        ws_bytes = L.llmq_gemm_workspace_bytes(M, N, K)
+        self.ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        self.ws_bytes = ws_bytes
+        self.L, self.abi = L, _abi
+        self.ops = 2 * M * N * K
+
+    def quant(self, stream):
+        return self.L.llmq_quant_i8_per_token(self.x.data_ptr(), self.abi.BF16, self.M, self.K, self.K,
+                                              self.qx.data_ptr(), self.a_scale.data_ptr(), self.abi.F32, stream)
+
+    def gemm(self, stream, acc_dump=None):
+        return self.L.llmq_gemm_w8a8(self.qx.data_ptr(), self.K, self.qweight.data_ptr(), self.K,
+                                     self.a_scale.data_ptr(), self.w_scale.data_ptr(), 1.0, None, None, 0, 0.0,
+                                     self.out.data_ptr(), self.abi.BF16, self.N, self.M, self.N, self.K,
+                                     acc_dump, self.ws.data_ptr(), self.ws.numel(), stream)
+
+    def launch(self, stream):
+        rc = self.quant(stream)
+        rc |= self.gemm(stream)
+        return rc
+
+
+def event_time_us(fn, stream_obj, reps):
+    """Average duration of fn() in microseconds from HIP events recorded on the launch stream."""
+    fn()
+    stream_obj.synchronize()
+    times = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream_obj)
+        fn()
+        e1.record(stream_obj)
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1) * 1e3)
+    return statistics.mean(times), min(times)
+
+
+def batch_time_us(fns, stream_obj, reps, rounds=5):
+    """Median over `rounds` of the per-launch time of back-to-back launches cycling through `fns`."""
+    for f in fns:
+        f()
+    stream_obj.synchronize()
+    per = []
+    for _ in range(rounds):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream_obj)
+        for i in range(reps):
+            fns[i % len(fns)]()
+        e1.record(stream_obj)
+        e1.synchronize()
+        per.append(e0.elapsed_time(e1) * 1e3 / reps)
+    return statistics.median(per)
+
+
+def build_w8a8_sweep(dev):
+    from llmqrt_amd import workloads as W
+    linears = []
+    for pi, (pname, (K, N)) in enumerate(W.QWEN2_7B_PROJ.items()):
+        qw, ws = W.int8_weights(N, K, W.seed_for(1, 100 + pi))
+        qw, ws = qw.to(dev), ws.to(dev)
+        for mi, M in enumerate(W.W8A8_M):
+            linears.append(W8A8Linear(f"{pname}_M{M}", M, K, N, qw, ws, W.seed_for(1, 10 * pi + mi), dev))
+    # big launches first so that the queue stays full while the host enqueues the small ones
+    linears.sort(key=lambda l: -l.ops)
+    return linears
+
+
+def cpu_baseline_and_parity(linears, dev):
+    """The oracle (dequantize-then-matmul, reference linear_sq.py:117-125) timed on the host cores
+    for the four projections at M = 2048, and used as the checker of the GPU results."""
+    from oracle import ref_math as R
+    sample = [l for l in linears if l.M == 2048]
+    stream = torch.cuda.current_stream().cuda_stream
+    total_ops, total_s, worst_rel, acc_exact = 0, 0.0, 0.0, True
+    for l in sample:
+        dump = torch.empty((l.M, l.N), dtype=torch.int32, device=dev)
+        l.quant(stream)
+        l.gemm(stream, dump.data_ptr())
+        torch.cuda.synchronize()
+        x_cpu, qw_cpu, ws_cpu = l.x.cpu(), l.qweight.cpu(), l.w_scale.cpu()
+        t0 = time.perf_counter()
+        qx, sx = R.quantize_activation_per_token_absmax(x_cpu)
+        y = R.w8a8_linear_naive(qx, sx, qw_cpu, ws_cpu, None, torch.bfloat16)
+        total_s += time.perf_counter() - t0
+        total_ops += l.ops
+        # checker (not timed): quantizer bit-exact, 64 sampled accumulator rows bit-exact, output tolerance
+        acc_exact &= torch.equal(l.qx.cpu(), qx) and torch.equal(l.a_scale.cpu(), sx.float().view(-1))
+        rows = torch.arange(0, l.M, l.M // 64)
+        acc_exact &= torch.equal(dump.cpu()[rows], R.int8_gemm_exact(qx[rows], qw_cpu))
+        rel = ((l.out.float().cpu() - y.float()).abs().max() / y.float().abs().max()).item()
+        worst_rel = max(worst_rel, rel)
+    return {
+        "value": round(total_ops / total_s / 1e12, 4), "unit": "TOPS", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": "per-token int8 quantizer + dequantize-then-matmul (torch fp32, oracle/ref_math.py) of the 4 "
+                  "Qwen2-7B projections at M=2048, 1 repetition, %d host threads of %d cores" %
+                  (torch.get_num_threads(), os.cpu_count()),
+        "seconds": round(total_s, 2),
+    }, {"int32_acc_and_quantizer_bit_exact": bool(acc_exact), "max_rel_err_vs_oracle": worst_rel, "tolerance": 1e-2}
+
+
+def details_fp8(dev):
+    from llmqrt_amd import _abi, workloads as W
+    L = _abi.lib()
+    stream_obj = torch.cuda.current_stream()
+    stream = stream_obj.cuda_stream
+    rows = []
+    for pi, (pname, (K, N)) in enumerate(W.QWEN2_7B_PROJ.items()):
+        wq, ws = W.fp8_weights(N, K, W.seed_for(2, 100 + pi))
+        wq, ws = wq.to(dev), ws.to(dev)
+        for mi, M in enumerate(W.FP8_M):
+            x = W.activations(M, K, W.seed_for(2, 10 * pi + mi)).to(dev)
+            xq = torch.empty((M, K), dtype=torch.float8_e4m3fn, device=dev)
+            xs = torch.empty((M,), dtype=torch.float32, device=dev)
+            out = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+            wsb = L.llmq_gemm_workspace_bytes(M, N, K)
+            wsp = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+
+            def quant():
+                L.llmq_quant_fp8_per_token(x.data_ptr(), _abi.BF16, M, K, K, xq.data_ptr(), xs.data_ptr(), stream)
+
+            def gemm():
+                L.llmq_gemm_fp8(xq.data_ptr(), _abi.E4M3, K, wq.data_ptr(), K, xs.data_ptr(), ws.data_ptr(), 1.0, None,
+                                None, 0, 0.0, out.data_ptr(), _abi.BF16, N, M, N, K, None, wsp.data_ptr(), wsp.numel(),
+                                stream)
+            quant()
+            t_gemm = batch_time_us([gemm], stream_obj, 20)
+            t_quant = batch_time_us([quant], stream_obj, 20)
+            tflops = 2 * M * N * K / t_gemm / 1e6
+            rows.append({"proj": pname, "M": M, "gemm_us": round(t_gemm, 2), "quant_us": round(t_quant, 2),
+                         "gemm_TFLOPS": round(tflops, 1), "pct_fp8_mfma_peak": round(100 * tflops / PEAK_FP8_TFLOPS, 2),
+                         "gemm_GBs": round(W.w8a8_gemm_bytes(M, N, K) / t_gemm / 1e3, 1)})
+    return rows
+
+
+def details_awq(dev):
+    from llmqrt_amd import _abi, workloads as W
+    L = _abi.lib()
+    stream_obj = torch.cuda.current_stream()
+    stream = stream_obj.cuda_stream
+    rows = []
+    for pi, (pname, (K, N)) in enumerate(W.QWEN2_7B_PROJ.items()):
+        qw, qz, sc = W.awq_weights(N, K, W.seed_for(3, 100 + pi))
+        wbytes = qw.numel() * 4 + qz.numel() * 4 + sc.numel() * 2
+        ncopies = max(2, -(-320 * 1024 * 1024 // wbytes))  # rotate through > 256 MB (Infinity Cache) of weights
+        copies = [(qw.to(dev).clone(), qz.to(dev).clone(), sc.to(dev).clone()) for _ in range(ncopies)]
+        for mi, M in enumerate(W.AWQ_M):
+            x = W.activations(M, K, W.seed_for(3, 10 * pi + mi), dtype=torch.float16, outliers=False).to(dev)
+            out = torch.empty((M, N), dtype=torch.float16, device=dev)
+            wsb = L.llmq_awq_gemm_workspace_bytes(M, N, K)
+            wsp = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+
+            def mk(c):
+                def f():
+                    L.llmq_awq_gemm(x.data_ptr(), K, c[0].data_ptr(), c[2].data_ptr(), c[1].data_ptr(), None,
+                                    out.data_ptr(), M, N, K, 128, wsp.data_ptr(), wsp.numel(), stream)
+                return f
+            fns = [mk(c) for c in copies]
+            t_rot = batch_time_us(fns, stream_obj, max(2 * ncopies, 40))
+            t_res = batch_time_us(fns[:1], stream_obj, 40)
+            b = W.awq_gemm_bytes(M, N, K)
+            rows.append({"proj": pname, "M": M, "us_hbm": round(t_rot, 2), "us_cache_resident": round(t_res, 2),
+                         "GBs_hbm": round(b / t_rot / 1e3, 1), "pct_hbm_peak": round(100 * b / t_rot / 1e3 / PEAK_HBM_GBS, 2),
+                         "GBs_cache_resident": round(b / t_res / 1e3, 1), "weight_copies_rotated": ncopies})
+        del copies
+    return rows
+
+
+def details_layer(dev):
+    """Config 4: one decoder layer's linears (qkv, o, gate_up, down) in W8A8 with SmoothQuant factors
+    (alpha = 0.5) folded into the preceding norm weight / the weights; prefill 2048 tokens and decode 32."""
+    from llmqrt_amd import _abi, workloads as W
+    stream_obj = torch.cuda.current_stream()
+    stream = stream_obj.cuda_stream
+    out = []
+    projs = list(W.QWEN2_7B_PROJ.items())
+    weights = {}
+    for pi, (pname, (K, N)) in enumerate(projs):
+        w = W.dense_weights(N, K, W.seed_for(4, 100 + pi))
+        calib = W.activations(256, K, W.seed_for(4, 200 + pi)).float()
+        s = W.smoothquant_factors(calib.abs().amax(0), w.abs().amax(0), 0.5)
+        ws = w * s.view(1, -1)                                   # weights absorb s
+        scale = ws.abs().amax(dim=1) / 127
+        qw = (ws / scale.view(-1, 1)).round().clamp(-128, 127).to(torch.int8)
+        weights[pname] = (qw.to(dev), scale.to(dev), s)
+    for M in (2048, 32):
+        lins = []
+        for pi, (pname, (K, N)) in enumerate(projs):
+            qw, scale, s = weights[pname]
+            lin = W8A8Linear(f"{pname}_M{M}", M, K, N, qw, scale, W.seed_for(4, 10 * pi), dev)
+            lin.x = (lin.x.float().cpu() / s.view(1, -1)).bfloat16().to(dev)   # activations arrive pre-divided by s
+            lins.append(lin)
+
+        def layer():
+            for l in lins:
+                l.launch(stream)
+        t = batch_time_us([layer], stream_obj, 10)
+        ops = sum(l.ops for l in lins)
+        per = {}
+        for l in lins:
+            per[l.name] = round(batch_time_us([lambda l=l: l.launch(stream)], stream_obj, 10), 2)
+        out.append({"M": M, "layer_linear_us": round(t, 2), "TOPS": round(ops / t / 1e6, 1), "per_linear_us": per})
+    return out
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: the quantized-linear path has no multi-GPU part "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    from llmqrt_amd import _abi, workloads as W
+    _abi.lib()
+    stream_obj = torch.cuda.current_stream()
+    stream = stream_obj.cuda_stream
+
+    linears = build_w8a8_sweep(dev)
+    total_ops = sum(l.ops for l in linears)
+    prefill = [l for l in linears if l.M >= 2048]
+
+    if args.roofline_only:
+        for l in prefill:
+            l.quant(stream)
+        torch.cuda.synchronize()
+        for _ in range(args.warmup):
+            for l in prefill:
+                l.gemm(stream)
+        torch.cuda.synchronize()
+        for _ in range(args.steps):
+            for l in prefill:
+                l.gemm(stream)
+        torch.cuda.synchronize()
+        print(json.dumps({"roofline_only": True, "launches_per_step": len(prefill), "steps": args.steps}))
+        return
+
+    def step():
+        rc = 0
+        for l in linears:
+            rc |= l.launch(stream)
+        return rc
+
+    for _ in range(args.warmup):
+        if step() != 0:
+            raise RuntimeError("a launch failed during warm-up")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = total_ops / (elapsed / args.steps) / 1e12
+
+    # ---- roofline of the dominant kernel: the int8 MFMA GEMM launches at the prefill shapes ----
+    ops_sum, us_sum, per_shape = 0, 0.0, []
+    for l in prefill:
+        t_mean, t_min = event_time_us(lambda l=l: l.gemm(stream), stream_obj, 10)
+        ops_sum += l.ops
+        us_sum += t_mean
+        per_shape.append({"shape": l.name, "us": round(t_mean, 2), "TOPS": round(l.ops / t_mean / 1e6, 1),
+                          "pct_int8_mfma_peak": round(100 * l.ops / t_mean / 1e6 / PEAK_INT8_TOPS, 2)})
+    achieved = ops_sum / us_sum / 1e6
+    roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": None,
+                "kernel": "gemm_tile_kernel<int8> at M in {2048, 8192} x {qkv, o, gate_up, down}",
+                "avg_launch_us": round(us_sum / len(prefill), 2), "launches": per_shape}
+
+    result = {
+        "metric": "W8A8/FP8 GEMM TOPS (% MFMA peak); W4A16 decode GB/s (% HBM peak), 1 GPU",
+        "value": round(value, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "configs[1]: SmoothQuant W8A8 sweep, Qwen2-7B qkv/o/gate_up/down x M in "
+                               "{1,16,128,2048,8192}, per-token int8 quantizer kernel + int8 MFMA GEMM with "
+                               "per-token x per-channel epilogue, bf16 in/out; value = sum(2MNK) / step time",
+                   "linears_per_step": len(linears), "ops_per_step": total_ops},
+        "pct_int8_mfma_peak": round(100 * value / PEAK_INT8_TOPS, 2),
+        "roofline": roofline,
+    }
+
+    if not args.no_details:
+        w8 = []
+        for l in sorted(linears, key=lambda l: (l.name.rsplit("_M", 1)[0], l.M)):
+            tg = batch_time_us([lambda l=l: l.gemm(stream)], stream_obj, 20)
+            tq = batch_time_us([lambda l=l: l.quant(stream)], stream_obj, 20)
+            tops = l.ops / tg / 1e6
+            w8.append({"shape": l.name, "gemm_us": round(tg, 2), "quant_us": round(tq, 2), "gemm_TOPS": round(tops, 1),
+                       "pct_int8_mfma_peak": round(100 * tops / PEAK_INT8_TOPS, 2),
+                       "gemm_GBs": round(W.w8a8_gemm_bytes(l.M, l.N, l.K) / tg / 1e3, 1),
+                       "quant_GBs": round(W.quant_bytes(l.M, l.K) / tq / 1e3, 1)})
+        result["details"] = {"w8a8": w8}
+
+    if not args.no_cpu:
+        cpu, parity = cpu_baseline_and_parity(linears, dev)
+        result["cpu_baseline"] = cpu
+        result["parity"] = parity
+    else:
+        result["cpu_baseline"] = None
+
+    if not args.no_details:
+        del linears, prefill
+        torch.cuda.empty_cache()
+        result["details"]["fp8"] = details_fp8(dev)
+        result["details"]["awq_w4a16"] = details_awq(dev)
+        result["details"]["layer_stack_w8a8"] = details_layer(dev)
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -225,14 +225,14 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
             for (int r = 0; r < 16; r++) {
                 const int m = m0 + wm * C::WTM + i * 32 + 8 * (r / 4) + 4 * khalf + (r % 4);
                 if (m >= M) continue;
+                const auto av = acc[i][j][r];  // scalar copy: bit_cast on a vector element reads lane 0 of the vector
+                const uint32_t raw = __builtin_bit_cast(uint32_t, av);
                 if (split) {
-                    reinterpret_cast<uint32_t*>(partials)[((int64_t)blockIdx.y * M + m) * N + n] =
-                        __builtin_bit_cast(uint32_t, acc[i][j][r]);
+                    reinterpret_cast<uint32_t*>(partials)[((int64_t)blockIdx.y * M + m) * N + n] = raw;
                 } else {
-                    if (acc_dump)
-                        reinterpret_cast<uint32_t*>(acc_dump)[(int64_t)m * N + n] = __builtin_bit_cast(uint32_t, acc[i][j][r]);
+                    if (acc_dump) reinterpret_cast<uint32_t*>(acc_dump)[(int64_t)m * N + n] = raw;
                     const float sa = ep.a_scale ? ep.a_scale[m] : 1.f;
-                    const float v = epi_value((float)acc[i][j][r], sa, sw, alpha, bb);
+                    const float v = epi_value((float)av, sa, sw, alpha, bb);
                     reinterpret_cast<uint16_t*>(out)[(int64_t)m * ldo + n] = to_out(v, ep.out_dtype);
                 }
             }

@@ -10,6 +10,12 @@ from oracle import ref_math as R
 
 pytestmark = pytest.mark.gpu
 REL_TOL = 1e-2
+# fp32 accumulators of the fp8 MFMA against an fp64 sum of the same exact products, relative to the
+# largest accumulator.  One v_mfma_f32_32x32x64_f8f6f4 adds its 64 products in a fixed-point window
+# below the largest of them (measured: errors up to ~5e-5 of the largest accumulator at K = 3584), the
+# same class of arithmetic as the reference's use_fast_accum=True tensor-core path; between
+# instructions the accumulation is plain fp32.
+FP8_ACC_TOL = 2e-4
 
 
 def rel_err(y, ref):
@@ -155,7 +161,7 @@ def test_fp8_rowwise(cuda, M, N, K):
                                       True, _acc_dump=dump)
     assert y.dtype == torch.bfloat16 and y.shape == (M, N)
     # fp32 accumulation of exact products: only the summation order differs from the fp64 sum
-    assert rel_err(dump, acc_ref) <= 1e-5
+    assert rel_err(dump, acc_ref) <= FP8_ACC_TOL
     assert rel_err(y, y_ref) <= REL_TOL
     assert rel_err(y, R.fp8_linear_naive(xq, xs, wq, ws, bias)) <= REL_TOL
     y_nb = cutlass_f8f8bf16_rowwise_sm89(xq.to(cuda), wq.to(cuda).t(), None, xs.to(cuda), ws.to(cuda).view(1, -1), True)
@@ -174,7 +180,7 @@ def test_fp8_every_tile_config(cuda, force_plan, splits):
         dump = torch.empty((M, N), dtype=torch.float32, device=cuda)
         y = cutlass_f8f8bf16_rowwise_sm89(xq.to(cuda), wq.to(cuda).t(), bias.to(cuda), xs.to(cuda),
                                           ws.to(cuda).view(1, -1), True, _acc_dump=dump)
-        assert rel_err(dump, acc_ref) <= 1e-5, f"cfg {cfg}"
+        assert rel_err(dump, acc_ref) <= FP8_ACC_TOL, f"cfg {cfg}"
         assert rel_err(y, y_ref) <= REL_TOL, f"cfg {cfg}"
 
 
