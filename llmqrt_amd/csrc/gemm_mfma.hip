@@ -65,6 +65,9 @@ struct GemmCfg {
     static constexpr int A_LOADS = BM * CPR / NT, B_LOADS = BN * CPR / NT;
     static constexpr int STAGE_CHUNKS = (BM + BN) * CPR;
     static constexpr size_t LDS_BYTES = 2u * STAGE_CHUNKS * 16u;
+    // Double-buffer the MFMA operand fragments (software pipeline LDS reads under MFMAs).  The fp8
+    // fragments are twice as wide; with two wavefronts per SIMD (256 registers each) they do not fit twice.
+    static constexpr bool PIPE = !(FP8 && NT > 256);
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be 32-aligned");
     static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "tile must split evenly over threads");
     static_assert(CPR == 4 || CPR == 8, "BK must be 64 or 128");
@@ -87,7 +90,7 @@ __device__ __forceinline__ void tile_coords(int bid, int nblk, int tiles_m, int 
     tn = (pid % width) / gsize;
 }
 
-template <class C>
+template <class C, bool KFULL>
 __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     const uint8_t* __restrict__ A, int64_t lda, const uint8_t* __restrict__ B, int64_t ldb,
     int M, int N, int K, int k_per_split, Epilogue ep, void* __restrict__ out, int64_t ldo,
@@ -120,10 +123,12 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     for (int i = 0; i < C::B_LOADS; i++) b_off[i] = min(ld_row + i * ROWS_STEP, N - 1 - n0) * (int)ldb;
     const int st_a = lds_chunk<C::CPR>(ld_row, ld_c);
     const int st_b = C::BM * C::CPR + st_a;
-    uint4 a_reg[C::A_LOADS], b_reg[C::B_LOADS];
-    auto load_tile = [&](int kt) {
+    uint4 ra[2][C::A_LOADS], rb[2][C::B_LOADS];  // two tiles in flight (register staging)
+    auto load_tile = [&](int kt, uint4* a_reg, uint4* b_reg) {
         const int koff = kt * C::BK;
-        const bool ok = ld_c * 16 < k_end - k_begin - koff;  // chunk inside this split's K range
+        // Tiles past the end of this split's K range load zeros (the main loop always runs an even
+        // number of tiles); inside the range a chunk is skipped only in the ragged last tile.
+        const bool ok = kt < ktiles && (KFULL || ld_c * 16 < k_end - k_begin - koff);
 #pragma unroll
         for (int i = 0; i < C::A_LOADS; i++)
             a_reg[i] = ok ? *reinterpret_cast<const uint4*>(a_base + a_off[i] + koff) : make_uint4(0, 0, 0, 0);
@@ -131,12 +136,18 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
         for (int i = 0; i < C::B_LOADS; i++)
             b_reg[i] = ok ? *reinterpret_cast<const uint4*>(b_base + b_off[i] + koff) : make_uint4(0, 0, 0, 0);
     };
-    auto store_tile = [&](int stage) {
+    auto store_tile = [&](int stage, const uint4* a_reg, const uint4* b_reg) {
         uint4* s = lds + stage * C::STAGE_CHUNKS;
 #pragma unroll
         for (int i = 0; i < C::A_LOADS; i++) s[st_a + i * ROWS_STEP * C::CPR] = a_reg[i];
 #pragma unroll
         for (int i = 0; i < C::B_LOADS; i++) s[st_b + i * ROWS_STEP * C::CPR] = b_reg[i];
+    };
+    // Block barrier that orders LDS traffic only: global loads stay in flight across it.
+    auto lds_barrier = [] {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     };
 
     acc_t acc[C::TM][C::TN];
@@ -151,90 +162,199 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     const int l32 = lane & 31, khalf = lane >> 5;  // row within the 32-row tile, K half of the lane
     const int a_row0 = wm * C::WTM + l32, b_row0 = wn * C::WTN + l32;
 
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-
-    for (int kt = 0; kt < ktiles; kt++) {
-        const bool more = kt + 1 < ktiles;
-        if (more) load_tile(kt + 1);
-        const uint4* sA = lds + (kt & 1) * C::STAGE_CHUNKS;
+    // MFMA operand fragments, double-buffered: while the matrix pipe works on one K sub-step the LDS
+    // already serves the reads of the next one (also across the block barrier, so the first reads of a
+    // freshly published stage overlap the last MFMAs of the previous tile).
+    using frag_t = typename std::conditional<C::FP8, v8i, v4i>::type;
+    frag_t fa[C::PIPE ? 2 : 1][C::TM], fb[C::PIPE ? 2 : 1][C::TN];
+    auto read_frags = [&](int stage, int ks, frag_t* af, frag_t* bf) {
+        const uint4* sA = lds + stage * C::STAGE_CHUNKS;
         const uint4* sB = sA + C::BM * C::CPR;
+        if constexpr (C::FP8) {
+            const int c0 = ks * 4 + khalf * 2;
 #pragma unroll
-        for (int ks = 0; ks < C::KSUB; ks++) {
-            if constexpr (C::FP8) {
-                v8i af[C::TM], bf[C::TN];
-                const int c0 = ks * 4 + khalf * 2;
+            for (int i = 0; i < C::TM; i++) {
+                const int row = a_row0 + i * 32;
+                const uint4 lo = sA[lds_chunk<C::CPR>(row, c0)], hi = sA[lds_chunk<C::CPR>(row, c0 + 1)];
+                af[i] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+            }
 #pragma unroll
-                for (int i = 0; i < C::TM; i++) {
-                    const int row = a_row0 + i * 32;
-                    const uint4 lo = sA[lds_chunk<C::CPR>(row, c0)], hi = sA[lds_chunk<C::CPR>(row, c0 + 1)];
-                    af[i] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-                }
+            for (int j = 0; j < C::TN; j++) {
+                const int row = b_row0 + j * 32;
+                const uint4 lo = sB[lds_chunk<C::CPR>(row, c0)], hi = sB[lds_chunk<C::CPR>(row, c0 + 1)];
+                bf[j] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+            }
+        } else {
+            const int c0 = ks * 2 + khalf;
 #pragma unroll
-                for (int j = 0; j < C::TN; j++) {
-                    const int row = b_row0 + j * 32;
-                    const uint4 lo = sB[lds_chunk<C::CPR>(row, c0)], hi = sB[lds_chunk<C::CPR>(row, c0 + 1)];
-                    bf[j] = v8i{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-                }
+            for (int i = 0; i < C::TM; i++) {
+                const uint4 v = sA[lds_chunk<C::CPR>(a_row0 + i * 32, c0)];
+                af[i] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+            }
 #pragma unroll
-                for (int i = 0; i < C::TM; i++)
-#pragma unroll
-                    for (int j = 0; j < C::TN; j++)
-                        acc[i][j] = (acc_t)__builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            af[i], bf[j], (v16f)acc[i][j], C::AFMT, 0, 0, 0, 0, 0);
-            } else {
-                v4i af[C::TM], bf[C::TN];
-                const int c0 = ks * 2 + khalf;
-#pragma unroll
-                for (int i = 0; i < C::TM; i++) {
-                    const uint4 v = sA[lds_chunk<C::CPR>(a_row0 + i * 32, c0)];
-                    af[i] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
-                }
-#pragma unroll
-                for (int j = 0; j < C::TN; j++) {
-                    const uint4 v = sB[lds_chunk<C::CPR>(b_row0 + j * 32, c0)];
-                    bf[j] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
-                }
-#pragma unroll
-                for (int i = 0; i < C::TM; i++)
-#pragma unroll
-                    for (int j = 0; j < C::TN; j++)
-                        acc[i][j] = (acc_t)__builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], (v16i)acc[i][j], 0, 0, 0);
+            for (int j = 0; j < C::TN; j++) {
+                const uint4 v = sB[lds_chunk<C::CPR>(b_row0 + j * 32, c0)];
+                bf[j] = v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
             }
         }
-        if (more) store_tile((kt + 1) & 1);
-        __syncthreads();
+    };
+    auto mfma_step = [&](const frag_t* af, const frag_t* bf) {
+#pragma unroll
+        for (int i = 0; i < C::TM; i++)
+#pragma unroll
+            for (int j = 0; j < C::TN; j++) {
+                if constexpr (C::FP8)
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[i][j], 0, C::AFMT,
+                                                                                0, 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
+            }
+    };
+    // Scheduling directive for one sub-step: issue the LDS reads of the next fragments one by one
+    // between the MFMAs of the current fragments (reads first), instead of after them.
+    auto interleave_reads_with_mfma = [] {
+        constexpr int kReads = (C::TM + C::TN) * (C::FP8 ? 2 : 1), kMfma = C::TM * C::TN;
+        constexpr int kPairs = kReads < kMfma ? kReads : kMfma;
+#pragma unroll
+        for (int n = 0; n < kPairs; n++) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one DS read
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        }
+        if (kReads > kPairs) __builtin_amdgcn_sched_group_barrier(0x100, kReads - kPairs, 0);
+        if (kMfma > kPairs) __builtin_amdgcn_sched_group_barrier(0x008, kMfma - kPairs, 0);
+    };
+    // One K tile: sub-steps 0 .. KSUB-2 read the next sub-step of the same stage; the last sub-step
+    // publishes the next tile (registers -> other stage), crosses the barrier and reads that stage's
+    // first sub-step.  `par` is the fragment-buffer parity on entry (compile-time).
+    auto tile_steps = [&](int stage, auto par_c, const uint4* a_reg, const uint4* b_reg) {
+        constexpr int par = decltype(par_c)::value;
+        if constexpr (!C::PIPE) {
+#pragma unroll
+            for (int ks = 0; ks < C::KSUB; ks++) {
+                read_frags(stage, ks, fa[0], fb[0]);
+                mfma_step(fa[0], fb[0]);
+            }
+            store_tile(stage ^ 1, a_reg, b_reg);
+            lds_barrier();
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < C::KSUB - 1; ks++) {
+                read_frags(stage, ks + 1, fa[(par + ks + 1) & 1], fb[(par + ks + 1) & 1]);
+                mfma_step(fa[(par + ks) & 1], fb[(par + ks) & 1]);
+                interleave_reads_with_mfma();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            store_tile(stage ^ 1, a_reg, b_reg);
+            lds_barrier();
+            read_frags(stage ^ 1, 0, fa[(par + C::KSUB) & 1], fb[(par + C::KSUB) & 1]);
+            mfma_step(fa[(par + C::KSUB - 1) & 1], fb[(par + C::KSUB - 1) & 1]);
+            interleave_reads_with_mfma();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // ---- main loop: tile kt is computed from LDS stage kt & 1 while tile kt+1 sits in registers
+    // and tile kt+2 is in flight from global memory.  Two tiles per iteration, no conditional
+    // compute: an odd tile count is padded with a zero tile -----------------------------------
+    load_tile(0, ra[0], rb[0]);
+    load_tile(1, ra[1], rb[1]);
+    store_tile(0, ra[0], rb[0]);
+    lds_barrier();
+    if constexpr (C::PIPE) read_frags(0, 0, fa[0], fb[0]);
+#pragma unroll 1
+    for (int kt = 0; kt < ktiles; kt += 2) {
+        load_tile(kt + 2, ra[0], rb[0]);
+        tile_steps(0, std::integral_constant<int, 0>{}, ra[1], rb[1]);
+        load_tile(kt + 3, ra[1], rb[1]);
+        tile_steps(1, std::integral_constant<int, C::KSUB & 1>{}, ra[0], rb[0]);
     }
 
-    // ---- epilogue: lane holds column n = l32, rows 8*(r/4) + 4*khalf + r%4 of each tile -----
+    // ---- epilogue.  The weights feed the MFMA row operand, so D is the transposed tile: a lane holds
+    // token m = l32 and, in register r, channel 8*(r/4) + 4*khalf + r%4 -> 4 consecutive channels per
+    // register quad.  After the dequant math the two half-waves exchange quads (v_permlane32_swap) so
+    // that every lane owns 8 consecutive channels of its token and stores them as one 16-byte vector.
     const bool split = gridDim.y > 1;
     const float alpha = ep.alpha * (ep.alpha_dev ? *ep.alpha_dev : 1.0f);
+    const bool out_vec = ((ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(out) & 15u) == 0);
+    const bool raw_vec = (N & 3) == 0;
 #pragma unroll
     for (int j = 0; j < C::TN; j++) {
-        const int n = n0 + wn * C::WTN + j * 32 + l32;
-        if (n >= N) continue;
-        float sw = 1.f, bb = 0.f;
-        if (!split) {
-            if (ep.w_scale) sw = ep.w_scale[n];
-            if (ep.bias) bb = ep.beta * load_as_f32(ep.bias, ep.bias_dtype, n);
+        const int nb = n0 + wn * C::WTN + j * 32;  // first channel of this 32-wide MFMA tile (wave-uniform)
+        if (nb >= N) continue;
+        const bool full = nb + 32 <= N;
+        float sw[16], bb[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int n = min(nb + 8 * (r / 4) + 4 * khalf + (r % 4), N - 1);
+            sw[r] = (!split && ep.w_scale) ? ep.w_scale[n] : 1.f;
+            bb[r] = (!split && ep.bias) ? ep.beta * load_as_f32(ep.bias, ep.bias_dtype, n) : 0.f;
         }
 #pragma unroll
         for (int i = 0; i < C::TM; i++) {
+            __builtin_amdgcn_sched_barrier(0);  // one tile at a time: keeps the accumulator copies short-lived
+            const int m = m0 + wm * C::WTM + i * 32 + l32;
+            const bool m_ok = m < M;
+            uint32_t raw[16];
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int m = m0 + wm * C::WTM + i * 32 + 8 * (r / 4) + 4 * khalf + (r % 4);
-                if (m >= M) continue;
-                const auto av = acc[i][j][r];  // scalar copy: bit_cast on a vector element reads lane 0 of the vector
-                const uint32_t raw = __builtin_bit_cast(uint32_t, av);
-                if (split) {
-                    reinterpret_cast<uint32_t*>(partials)[((int64_t)blockIdx.y * M + m) * N + n] = raw;
-                } else {
-                    if (acc_dump) reinterpret_cast<uint32_t*>(acc_dump)[(int64_t)m * N + n] = raw;
-                    const float sa = ep.a_scale ? ep.a_scale[m] : 1.f;
-                    const float v = epi_value((float)av, sa, sw, alpha, bb);
-                    reinterpret_cast<uint16_t*>(out)[(int64_t)m * ldo + n] = to_out(v, ep.out_dtype);
+                const auto av = acc[i][j][r];  // scalar copy first: bit_cast of a vector element misreads
+                raw[r] = __builtin_bit_cast(uint32_t, av);
+            }
+            if (split || acc_dump) {
+                uint32_t* dst = split ? reinterpret_cast<uint32_t*>(partials) + ((int64_t)blockIdx.y * M + m) * N
+                                      : reinterpret_cast<uint32_t*>(acc_dump) + (int64_t)m * N;
+                if (m_ok) {
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const int n = nb + 8 * g + 4 * khalf;
+                        if (full && raw_vec) {
+                            *reinterpret_cast<uint4*>(dst + n) = make_uint4(raw[4 * g], raw[4 * g + 1], raw[4 * g + 2], raw[4 * g + 3]);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (n + e < N) dst[n + e] = raw[4 * g + e];
+                        }
+                    }
                 }
+                if (split) continue;
+            }
+            const float sa = (ep.a_scale && m_ok) ? ep.a_scale[m] : 1.f;
+            uint32_t pk[4][2];  // pk[g] = 4 output elements (channels 8g + 4*khalf .. +3)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                uint16_t h[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const auto av = acc[i][j][4 * g + e];
+                    h[e] = to_out(epi_value((float)av, sa, sw[4 * g + e], alpha, bb[4 * g + e]), ep.out_dtype);
+                }
+                pk[g][0] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+                pk[g][1] = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+            }
+            uint16_t* orow = reinterpret_cast<uint16_t*>(out) + (int64_t)m * ldo;
+            if (full && out_vec) {
+                // lower half-wave keeps quads 0,1 and receives the upper half's quads 0,1 (channels +4..+7);
+                // upper half-wave keeps quads 2,3 and receives the lower half's quads 2,3
+#pragma unroll
+                for (int g = 0; g < 2; g++) {
+#pragma unroll
+                    for (int x = 0; x < 2; x++) {
+                        const auto sw2 = __builtin_amdgcn_permlane32_swap(pk[g][x], pk[g + 2][x], false, false);
+                        pk[g][x] = sw2[0];
+                        pk[g + 2][x] = sw2[1];
+                    }
+                    if (m_ok)
+                        *reinterpret_cast<uint4*>(orow + nb + 16 * khalf + 8 * g) =
+                            make_uint4(pk[g][0], pk[g][1], pk[g + 2][0], pk[g + 2][1]);
+                }
+            } else if (m_ok) {
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int n = nb + 8 * g + 4 * khalf + e;
+                        if (n < N) orow[n] = (uint16_t)(pk[g][e >> 1] >> (16 * (e & 1)));
+                    }
             }
         }
     }
@@ -306,26 +426,33 @@ Plan make_plan(int64_t M, int64_t N, int64_t K) {
         const int kps = cdiv(cdiv(K, osp), s.bk) * s.bk;
         return Plan{ocfg < kNumShapes ? ocfg : kNumShapes - 1, cdiv(K, kps), kps};
     }
-    Plan best{0, 1, (int)K};
+    // Cost model calibrated on MI355X (microseconds): a CU runs `per_cu` blocks at a time, a block needs
+    // t_tile per 64 bytes of K plus a fixed prologue/epilogue cost; blocks execute in rounds over the
+    // 256 CUs.  Split-K adds a second kernel and the round trip of the fp32/int32 partials.
+    struct Model { int cfg, per_cu; double t_tile, fixed; };
+    static const Model kModels[] = {
+        {1, 1, 0.98, 14.5},   // 256x256, 8 waves
+        {2, 1, 0.665, 14.4},  // 256x128
+        {3, 2, 0.636, 11.1},  // 128x128 (two blocks per CU, times are per resident pair)
+        {4, 3, 0.40, 7.0},    // 64x128
+        {5, 4, 0.30, 6.0},    // 32x128
+    };
+    Plan best{1, 1, (int)K};
     double best_t = 1e300;
-    for (int c = 0; c < kNumShapes; c++) {
-        const TileShape s = kShapes[c];
-        if (c == 0) continue;                                             // kept for tuning runs only
-        if (s.bm > 32 && M <= s.bm / 2 && c != kNumShapes - 1) continue;  // mostly padding
+    for (const Model& md : kModels) {
+        const TileShape s = kShapes[md.cfg];
+        if (M > 128 && md.cfg >= 4) continue;                 // skinny tiles are for decode-sized M
+        if (md.cfg < 5 && M <= s.bm / 2) continue;            // mostly padding
         const int64_t tiles = (int64_t)cdiv(M, s.bm) * cdiv(N, s.bn);
-        const int max_split = (int)std::min<int64_t>(16, K / (4 * s.bk) > 0 ? K / (4 * s.bk) : 1);
-        for (int sp = 1; sp <= max_split; sp *= 2) {
+        for (int sp = 1; sp <= 16; sp++) {
+            if (sp > 1 && (K / sp < 512 || (int64_t)M * N * sp > (int64_t)64 << 20)) break;
             const int kps = cdiv(cdiv(K, sp), s.bk) * s.bk;
             const int eff_sp = cdiv(K, kps);
-            const int64_t blocks = tiles * eff_sp;
-            const int per_cu = (s.bm * s.bn >= 256 * 128) ? 1 : 2;  // resident blocks per CU
-            const double rounds = (double)cdiv(blocks, (int64_t)kNumCu * per_cu);
-            // per block: MFMA cycles at 4 SIMDs (2048 op/clk each) vs bytes streamed at ~20 B/clk/CU
-            const double mfma = 2.0 * s.bm * s.bn * kps / (4 * 2048.0) * per_cu;
-            const double bytes = (double)(s.bm + s.bn) * kps / 24.0 * per_cu;
-            double t = rounds * (std::max(mfma, bytes) + 2000.0);
-            if (eff_sp > 1) t += 6000.0 + (double)M * N * eff_sp * 4.0 / (kNumCu * 16.0);
-            if (t < best_t) { best_t = t; best = Plan{c, eff_sp, kps}; }
+            if (eff_sp != sp) continue;
+            const double rounds = (double)cdiv(tiles * sp, (int64_t)kNumCu * md.per_cu);
+            double t = rounds * (kps / 64.0 * md.t_tile + md.fixed);
+            if (sp > 1) t += 6.0 + (double)M * N * sp * 8.0 / 3.0e6;
+            if (t < best_t) { best_t = t; best = Plan{md.cfg, sp, kps}; }
         }
     }
     return best;
@@ -335,12 +462,20 @@ template <class C>
 int launch_cfg(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, int M, int N, int K, const Plan& p,
                const Epilogue& ep, void* out, int64_t ldo, void* acc_dump, void* ws, hipStream_t st) {
     if (C::LDS_BYTES > 65536u &&
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<C>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES) != hipSuccess)
+        (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<C, true>),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES) != hipSuccess ||
+         hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<C, false>),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES) != hipSuccess))
         return LLMQ_ERR_LAUNCH;
     const int tiles = cdiv(M, C::BM) * cdiv(N, C::BN);
-    hipLaunchKernelGGL((gemm_tile_kernel<C>), dim3(tiles, p.splits), dim3(C::NT), C::LDS_BYTES, st, A, lda, B, ldb,
-                       M, N, K, p.k_per_split, ep, out, ldo, acc_dump, ws);
+    // every split covers whole K tiles -> the loads need no K predicate
+    const bool kfull = (K % C::BK == 0) && (p.k_per_split % C::BK == 0);
+    if (kfull)
+        hipLaunchKernelGGL((gemm_tile_kernel<C, true>), dim3(tiles, p.splits), dim3(C::NT), C::LDS_BYTES, st, A, lda, B,
+                           ldb, M, N, K, p.k_per_split, ep, out, ldo, acc_dump, ws);
+    else
+        hipLaunchKernelGGL((gemm_tile_kernel<C, false>), dim3(tiles, p.splits), dim3(C::NT), C::LDS_BYTES, st, A, lda,
+                           B, ldb, M, N, K, p.k_per_split, ep, out, ldo, acc_dump, ws);
     return launch_status();
 }
 

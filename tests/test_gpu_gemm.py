@@ -65,11 +65,13 @@ def test_w8a8_per_channel(cuda, M, N, K):
     assert rel_err(y, naive) <= REL_TOL
 
 
+# K = 1040 gives an odd number of K tiles plus a 16-byte tail, 1024 an even number, 128 / 64 a single tile
+@pytest.mark.parametrize("K", [1040, 1024, 128, 64, 384])
 @pytest.mark.parametrize("splits", [1, 2, 3])
-def test_w8a8_every_tile_config(cuda, force_plan, splits):
+def test_w8a8_every_tile_config(cuda, force_plan, splits, K):
     """Each tile configuration and the split-K path, on a ragged shape; accumulators bit-exact."""
     from llmqrt_amd.sq_fp8_kernels import w8a8_int8_linear_bbf16_obf16_per_channel
-    M, N, K = 300, 392, 1040
+    M, N = 300, 392
     qx, sx, qw, sw, bias = _int8_problem(M, N, K, 7)
     acc_ref = R.int8_gemm_exact(qx, qw)
     y_ref = R.w8a8_epilogue_per_token_per_channel(acc_ref, sx, sw, bias, torch.bfloat16)
@@ -168,10 +170,11 @@ def test_fp8_rowwise(cuda, M, N, K):
     assert rel_err(y_nb, R.fp8_epilogue_rowwise(acc_ref, xs, ws, None)) <= REL_TOL
 
 
-@pytest.mark.parametrize("splits", [1, 2])
-def test_fp8_every_tile_config(cuda, force_plan, splits):
+@pytest.mark.parametrize("K", [1040, 1024, 128, 64, 384])
+@pytest.mark.parametrize("splits", [1, 2, 3])
+def test_fp8_every_tile_config(cuda, force_plan, splits, K):
     from llmqrt_amd.sq_fp8_kernels import cutlass_f8f8bf16_rowwise_sm89
-    M, N, K = 300, 392, 1040
+    M, N = 300, 392
     xq, xs, wq, ws, bias = _fp8_problem(M, N, K, 9)
     acc_ref = R.fp8_gemm_acc(xq, wq)
     y_ref = R.fp8_epilogue_rowwise(acc_ref, xs, ws, bias)
