@@ -142,13 +142,21 @@ int llmq_gemm_num_configs(void);
 /* out[m,n] = fp16( sum_k x[m,k] * fp16((q[k,n] - z[k/G,n]) * s[k/G,n]) + bias[n] ), fp32
  * accumulation in a fixed order (deterministic, unlike the reference's fp16 atomics).
  * x: fp16 [M,K] (ldx >= K, K % 32 == 0); out: fp16 [M,N] contiguous; bias: fp16 [N] or NULL.
- * workspace: >= llmq_awq_gemm_workspace_bytes(M,N,K) bytes. */
+ * For M <= 16 and group 128 the weights enter the matrix core unrounded (exact (q - z) * s in
+ * fp32) instead of rounded to fp16 first; both are within 1e-2 of the dequantize-then-matmul math.
+ * workspace: >= llmq_awq_gemm_workspace_bytes(M,N,K) bytes, 16-byte aligned, contents irrelevant. */
 int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight, const void* scales,
                   const int32_t* qzeros, const void* bias, void* out,
                   int64_t M, int64_t N, int64_t K, int64_t group,
                   void* workspace, size_t workspace_bytes, llmq_stream_t stream);
 
 size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/* Tuning / test hook with no counterpart in the reference: force the words-per-lane variant
+ * (v = 1 or 2; 0 = heuristic), the cross-block K split (0 = heuristic) and the wavefronts per
+ * block along K of the decode kernel (4 or 8; 0 = heuristic) of llmq_awq_gemm for every later
+ * call of this process.  Process-global, not thread-safe. */
+int llmq_awq_force_plan(int v, int splits, int k_waves);
 
 /* out: fp16 [K, N] contiguous = fp16(q - z) * s, bit-exact with
  * utils/packing_utils.py:65-80 (dequantize_gemm). */

@@ -39,6 +39,7 @@ SIGNATURES = {
     "llmq_gemm_num_configs": (_int, []),
     "llmq_awq_gemm": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
     "llmq_awq_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "llmq_awq_force_plan": (_int, [_int, _int, _int]),
     "llmq_awq_dequant": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
 }
 

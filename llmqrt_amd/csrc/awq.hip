@@ -58,7 +58,8 @@ __global__ __launch_bounds__(kBlockWaves * kWave) void awq_gemm_kernel(
     constexpr int NACC = MT * V * 8;
     __shared__ float4 red[NACC * kWave];
 
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // wave-uniform: keeps the K-range branches scalar
     const int li = lane & 15, kb = lane >> 4;
     const int Nw = N >> 3;
     const int cw = blockIdx.x * (16 * V) + V * li;  // first word column of this lane
@@ -81,8 +82,12 @@ __global__ __launch_bounds__(kBlockWaves * kWave) void awq_gemm_kernel(
     h2 cz[V][8], s2[V][8];  // per-group constants: -(bias+zero) and the scale, both halves equal
     int cur_g = -1;
 
-    wvec wcur[8], wnext[8];
-    uint4 xcur[MT], xnext[MT];
+    // Chunk ring: 4 chunks of packed words (+ their activations) are in flight per wavefront, so a
+    // chunk's loads are issued three chunk-times before they are consumed; the zeros / scales of the
+    // next group are fetched while the current group is being processed.
+    constexpr int RING = 4;
+    wvec wr[RING][8];
+    uint4 xr[RING][MT];
     auto load_chunk = [&](int c, wvec* wdst, uint4* xdst) {
         const int k0 = c * kChunkK + 8 * kb;
         const uint32_t* wp = qw + (int64_t)k0 * Nw + cwc;
@@ -94,19 +99,38 @@ __global__ __launch_bounds__(kBlockWaves * kWave) void awq_gemm_kernel(
             xdst[a] = m < M ? *reinterpret_cast<const uint4*>(x + (int64_t)m * ldx + k0) : make_uint4(0, 0, 0, 0);
         }
     };
+    wvec zv_next;
+    uint4 sv_next[V];
+    auto load_group = [&](int g) {
+        zv_next = *reinterpret_cast<const wvec*>(qz + (int64_t)g * Nw + cwc);
+#pragma unroll
+        for (int t = 0; t < V; t++)
+            sv_next[t] = *reinterpret_cast<const uint4*>(scales + (int64_t)g * N + 8 * (cwc + t));
+    };
+    // 0x64006400 kept in a register the optimizer cannot see through, so that (u & mask) | magic is one
+    // v_and_or_b32 (a VOP3 instruction may carry only one literal)
+    uint32_t magic = 0x64006400u;
+    asm volatile("" : "+v"(magic));
 
-    if (c0 < c1) load_chunk(c0, wcur, xcur);
-    for (int c = c0; c < c1; c++) {
-        if (c + 1 < c1) load_chunk(c + 1, wnext, xnext);
+    const int ngroups = K / G;
+    if (c0 < c1) load_group((c0 * kChunkK) / G);
+#pragma unroll
+    for (int u = 0; u < RING; u++)
+        if (c0 + u < c1) load_chunk(c0 + u, wr[u], xr[u]);
+
+    auto process = [&](int c, const wvec* wcur, const uint4* xcur) {
         const int g = (c * kChunkK) / G;
         if (g != cur_g) {
             cur_g = g;
-            const wvec zv = *reinterpret_cast<const wvec*>(qz + (int64_t)g * Nw + cwc);
+            const wvec zv = zv_next;
+            uint4 sv[V];
+#pragma unroll
+            for (int t = 0; t < V; t++) sv[t] = sv_next[t];
+            if (g + 1 < ngroups && ((g + 1) * G) / kChunkK < c1) load_group(g + 1);
 #pragma unroll
             for (int t = 0; t < V; t++) {
                 const uint32_t zw = word_of<V>(zv, t);
-                const uint4 sv = *reinterpret_cast<const uint4*>(scales + (int64_t)g * N + 8 * (cwc + t));
-                const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w};
+                const uint32_t sw[4] = {sv[t].x, sv[t].y, sv[t].z, sv[t].w};
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
                     constexpr uint32_t kLoBase = 0xE400u, kHiBase = 0xD400u;  // -(1024), -(64) as fp16 bits
@@ -135,12 +159,12 @@ __global__ __launch_bounds__(kBlockWaves * kWave) void awq_gemm_kernel(
                     const uint32_t u = __builtin_amdgcn_perm(w1, w0, sel);  // byte0 <- w0, byte2 <- w1
                     h2 d;
                     if (p & 1) {
-                        const h2 h = __builtin_bit_cast(h2, (u & 0x00F000F0u) | 0x64006400u);  // 1024 + 16 q
+                        const h2 h = __builtin_bit_cast(h2, (u & 0x00F000F0u) | magic);  // 1024 + 16 q
                         const h2 k16 = {(_Float16)0.0625f, (_Float16)0.0625f};
-                        d = __builtin_elementwise_fma(h, k16, cz[t][j]);                       // q - z, exact
+                        d = __builtin_elementwise_fma(h, k16, cz[t][j]);                 // q - z, exact
                     } else {
-                        const h2 h = __builtin_bit_cast(h2, (u & 0x000F000Fu) | 0x64006400u);  // 1024 + q
-                        d = h + cz[t][j];                                                      // q - z, exact
+                        const h2 h = __builtin_bit_cast(h2, (u & 0x000F000Fu) | magic);  // 1024 + q
+                        d = h + cz[t][j];                                                // q - z, exact
                     }
                     ar[pr] = __builtin_bit_cast(uint32_t, d * s2[t][j]);  // fp16((q - z) * s), one rounding
                 }
@@ -150,10 +174,16 @@ __global__ __launch_bounds__(kBlockWaves * kWave) void awq_gemm_kernel(
                     acc[a][t][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af, xb[a], acc[a][t][j], 0, 0, 0);
             }
         }
+    };
+
+    for (int c = c0; c < c1; c += RING) {
 #pragma unroll
-        for (int r = 0; r < 8; r++) wcur[r] = wnext[r];
-#pragma unroll
-        for (int a = 0; a < MT; a++) xcur[a] = xnext[a];
+        for (int u = 0; u < RING; u++) {
+            if (c + u < c1) {
+                process(c + u, wr[u], xr[u]);
+                if (c + u + RING < c1) load_chunk(c + u + RING, wr[u], xr[u]);
+            }
+        }
     }
 
     // ---- sum the 4 wavefronts in wave order through LDS ---------------------------------------
@@ -224,6 +254,221 @@ __global__ __launch_bounds__(kBlockWaves * kWave) void awq_gemm_kernel(
     }
 }
 
+// Decode kernel (M <= 16, group size 128).  Same streaming scheme, with the scale and the zero point
+// moved out of the per-weight work.  The raw nibbles go to the matrix core as fp16 SUBNORMALS:
+// (u & 0x000F000F) read as two fp16 values is q * 2^-24 (a high nibble, u & 0x00F000F0, is
+// 16 q * 2^-24); their products with fp16 activations are exact in the fp32 accumulator.  Per
+// quantization group and output channel
+//   y[m,n] += s[n] * 2^24 * acc[m,n]  -  s[n] * z[n] * xsum[m],
+// where xsum[m] = sum_k x[m,k] over the group comes from one extra MFMA against a vector of ones.
+// Unpacking is one v_perm_b32 per two k-pairs plus one v_and_b32 per pair (0.75 VALU op per weight),
+// and two FMAs per group and output.  The tokens are the MFMA rows and the lane's own word columns the
+// MFMA columns, so each lane needs exactly the zeros word and the 8 scales of the columns it streams.
+// Weights are never rounded to fp16 here (the reference dequantizer rounds (q - z) * s once): the
+// result is the exact-weight product, well inside the tolerance of that math.
+//
+// Work unit = one group = 4 chunks of 32 k.  The loop body is branch-free: every load is issued
+// unconditionally (indices clamped to the wavefront's last group) so that the compiler can count the
+// loads in flight and wait only for the oldest ring slot; 4 chunks (+ the next group's zeros/scales)
+// stay in flight per wavefront.
+template <int V, int KW>
+__global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, const uint32_t* __restrict__ qw,
+    const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qz, const uint16_t* __restrict__ bias,
+    uint16_t* __restrict__ out, float* __restrict__ partials, int M, int N, int K) {
+    typedef typename WordVec<V>::type wvec;
+    constexpr int G = 128, RING = G / kChunkK, NACC = V * 8;
+    __shared__ float4 red[(KW / 2) * NACC * kWave];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // scalar: keeps the loop bounds uniform
+    const int li = lane & 15, kb = lane >> 4;
+    const int Nw = N >> 3;
+    // Column tile of this block.  Consecutive block ids are dealt round-robin to the 8 XCDs; give each
+    // XCD a contiguous range of tiles instead, so that the two 64-byte halves of a cache line (adjacent
+    // tiles when V == 1) are fetched through the same L2.
+    int tile = blockIdx.x;
+    {
+        const int nb = gridDim.x, q = nb / 8, r = nb % 8, xcd = tile % 8, local = tile / 8;
+        tile = xcd < r ? xcd * (q + 1) + local : r * (q + 1) + (xcd - r) * q + local;
+    }
+    const int cw = tile * (16 * V) + V * li;  // first word column of this lane
+    const bool col_ok = cw < Nw;
+    const int cwc = col_ok ? cw : 0;
+
+    // Groups are dealt cyclically over all gridDim.y * KW wavefronts that share a column tile: at any
+    // moment they work on neighbouring groups, so the whole grid sweeps one compact window of rows
+    // down the matrix (DRAM pages are used up while open) instead of gridDim.y * KW distant ones.
+    const int ngroups = K / G;
+    const int gstride = (int)gridDim.y * KW;
+    const int g0 = (int)blockIdx.y * KW + wave;
+
+    v4f y[V][8], accg[V][8], xs = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < V; t++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            y[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+            accg[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+        }
+
+    if (g0 < ngroups) {
+        wvec wr[RING][8];
+        uint4 xr[RING];
+        uint32_t voff[8];  // loop-invariant row offsets; the chunk base is wave-uniform
+#pragma unroll
+        for (int r = 0; r < 8; r++) voff[r] = (uint32_t)(((8 * kb + r) * Nw + cwc) * 4);
+        const uint32_t xoff = (uint32_t)((min(li, M - 1) * (int)ldx + 8 * kb) * 2);
+        // loads past the last group of this wavefront re-read that group (results unused): no branches
+        auto load_chunk = [&](int g, int u, wvec* wdst, uint4& xdst) {
+            const int c = (g < ngroups ? g : g - gstride) * RING + u;
+            const uint8_t* wbase = reinterpret_cast<const uint8_t*>(qw) + (int64_t)c * kChunkK * Nw * 4;
+#pragma unroll
+            for (int r = 0; r < 8; r++) wdst[r] = *reinterpret_cast<const wvec*>(wbase + voff[r]);
+            xdst = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(x) + (int64_t)c * kChunkK * 2 + xoff);
+        };
+        wvec z_cur, z_next;
+        uint4 s_cur[V], s_next[V];
+        auto load_group = [&](int g) {
+            g = g < ngroups ? g : g - gstride;
+            z_next = *reinterpret_cast<const wvec*>(qz + (int64_t)g * Nw + cwc);
+#pragma unroll
+            for (int t = 0; t < V; t++)
+                s_next[t] = *reinterpret_cast<const uint4*>(scales + (int64_t)g * N + 8 * (cwc + t));
+        };
+        const h8 ones = {(_Float16)1.f, (_Float16)1.f, (_Float16)1.f, (_Float16)1.f,
+                         (_Float16)1.f, (_Float16)1.f, (_Float16)1.f, (_Float16)1.f};
+        const bool row_ok = li < M;
+
+        // same issue order as in the loop (group, slot 0..3), pinned, so that the wait counts the compiler
+        // derives at the loop head are those of the steady state
+        load_group(g0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < RING; u++) {
+            load_chunk(g0, u, wr[u], xr[u]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+#pragma unroll 1
+        for (int g = g0; g < ngroups; g += gstride) {
+            z_cur = z_next;
+#pragma unroll
+            for (int t = 0; t < V; t++) s_cur[t] = s_next[t];
+            load_group(g + gstride);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < RING; u++) {
+                uint4 xv = xr[u];
+                if (!row_ok) xv = make_uint4(0, 0, 0, 0);
+                const h8 xb = __builtin_bit_cast(h8, xv);
+                xs = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb, ones, xs, 0, 0, 0);
+#pragma unroll
+                for (int t = 0; t < V; t++) {
+#pragma unroll
+                    for (int bsel = 0; bsel < 4; bsel++) {  // byte of the word: nibbles 2*bsel (low), 2*bsel+1 (high)
+                        const uint32_t sel = (uint32_t)bsel | 0x0c00u | ((uint32_t)(4 + bsel) << 16) | 0x0c000000u;
+                        uint32_t lo[4], hi[4];
+#pragma unroll
+                        for (int pr = 0; pr < 4; pr++) {
+                            const uint32_t w0 = word_of<V>(wr[u][2 * pr], t), w1 = word_of<V>(wr[u][2 * pr + 1], t);
+                            const uint32_t uu = __builtin_amdgcn_perm(w1, w0, sel);  // byte0 <- w0, byte2 <- w1
+                            lo[pr] = uu & 0x000F000Fu;                               // q * 2^-24 as fp16 subnormals
+                            hi[pr] = uu & 0x00F000F0u;                               // 16 q * 2^-24
+                        }
+                        constexpr int kColOfNibble[8] = {0, 2, 4, 6, 1, 3, 5, 7};  // logical column of nibble p
+                        const int jl = kColOfNibble[2 * bsel], jh = kColOfNibble[2 * bsel + 1];
+                        const h8 bl = __builtin_bit_cast(h8, v4i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3]});
+                        const h8 bh = __builtin_bit_cast(h8, v4i{(int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]});
+                        accg[t][jl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb, bl, accg[t][jl], 0, 0, 0);
+                        accg[t][jh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb, bh, accg[t][jh], 0, 0, 0);
+                    }
+                }
+                // keep the issue order: this slot's refill goes out only now, and nothing of the next
+                // chunk is scheduled above it (the waits then cover only the oldest slot)
+                __builtin_amdgcn_sched_barrier(0);
+                load_chunk(g + gstride, u, wr[u], xr[u]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // y += s * 2^24 * acc - s * z * xsum for this group; the group accumulators restart at 0
+#pragma unroll
+            for (int t = 0; t < V; t++) {
+                const uint32_t zw = word_of<V>(z_cur, t);
+                const uint32_t sw[4] = {s_cur[t].x, s_cur[t].y, s_cur[t].z, s_cur[t].w};
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int p = rev_nibble(j);
+                    const float zf = (float)((zw >> (4 * p)) & 0xFu);
+                    const float sf = Lo<LLMQ_F16>::to_f32((uint16_t)((j & 1) ? (sw[j >> 1] >> 16) : (sw[j >> 1] & 0xffffu)));
+                    const float s1 = sf * ((p & 1) ? 1048576.0f : 16777216.0f);  // 2^20 for 16 q, 2^24 for q
+                    const float sz = -sf * zf;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        y[t][j][r] = fmaf(s1, accg[t][j][r], fmaf(sz, xs[r], y[t][j][r]));
+                        accg[t][j][r] = 0.f;
+                    }
+                }
+            }
+            xs = v4f{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+
+    // ---- sum the KW wavefronts through LDS: a fixed binary tree (upper half adds into lower half) -----
+#pragma unroll
+    for (int half = KW / 2; half >= 1; half /= 2) {
+        __syncthreads();
+        if (wave >= half && wave < 2 * half) {
+#pragma unroll
+            for (int t = 0; t < V; t++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const v4f v = y[t][j];
+                    red[((wave - half) * NACC + t * 8 + j) * kWave + lane] = make_float4(v[0], v[1], v[2], v[3]);
+                }
+        }
+        __syncthreads();
+        if (wave < half) {
+#pragma unroll
+            for (int t = 0; t < V; t++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float4 v = red[(wave * NACC + t * 8 + j) * kWave + lane];
+                    y[t][j] += v4f{v.x, v.y, v.z, v.w};
+                }
+        }
+    }
+    if (wave != 0 || !col_ok) return;
+
+    // ---- store: lane (word column li, quarter kb) holds tokens 4*kb + r for its 8*V channels -------
+    const bool split = gridDim.y > 1;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int m = 4 * kb + r;
+        if (m >= M) continue;
+#pragma unroll
+        for (int t = 0; t < V; t++) {
+            const int n = 8 * (cw + t);
+            if (split) {
+                float4* dst = reinterpret_cast<float4*>(partials + ((int64_t)blockIdx.y * M + m) * N + n);
+                dst[0] = make_float4(y[t][0][r], y[t][1][r], y[t][2][r], y[t][3][r]);
+                dst[1] = make_float4(y[t][4][r], y[t][5][r], y[t][6][r], y[t][7][r]);
+            } else {
+                uint32_t o[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    float lo = y[t][2 * j][r], hi = y[t][2 * j + 1][r];
+                    if (bias) {
+                        lo = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(lo)) + Lo<LLMQ_F16>::to_f32(bias[n + 2 * j]);
+                        hi = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(hi)) + Lo<LLMQ_F16>::to_f32(bias[n + 2 * j + 1]);
+                    }
+                    o[j] = (uint32_t)Lo<LLMQ_F16>::from_f32(lo) | ((uint32_t)Lo<LLMQ_F16>::from_f32(hi) << 16);
+                }
+                *reinterpret_cast<uint4*>(out + (int64_t)m * N + n) = make_uint4(o[0], o[1], o[2], o[3]);
+            }
+        }
+    }
+}
+
 // Cross-block split-K finish: sum partials in split order, round to fp16, add bias.
 __global__ __launch_bounds__(256) void awq_finish_kernel(const float* __restrict__ partials, int splits, int64_t total,
                                                          int N, const uint16_t* __restrict__ bias,
@@ -273,22 +518,47 @@ struct AwqPlan { int v, mt, splits, chunks_per_block; };
 
 inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
+int g_force_v = 0, g_force_splits = 0, g_force_kw = 0;  // tuning hook (llmq_awq_force_plan)
+
+// Generic kernel (any group size, up to 64 tokens): 4 wavefronts split the block's K range.
 AwqPlan make_awq_plan(int64_t M, int64_t N, int64_t K) {
     AwqPlan p;
     p.mt = cdiv(M, 16);
     const int Nw = (int)(N / 8);
-    p.v = (p.mt == 1 && Nw % 2 == 0 && N >= 16384) ? 2 : 1;
+    p.v = 1;
+    if (g_force_v == 2 && p.mt == 1 && Nw % 2 == 0) p.v = 2;
     const int ntiles = cdiv(Nw, 16 * p.v);
     const int chunks = (int)(K / kChunkK);
     // aim at ~2 blocks per CU; every wavefront should keep at least 4 chunks
-    int splits = cdiv(512, ntiles);
+    int splits = g_force_splits > 0 ? g_force_splits : cdiv(512, ntiles);
     const int max_splits = chunks / (4 * kBlockWaves) > 0 ? chunks / (4 * kBlockWaves) : 1;
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
-    p.chunks_per_block = cdiv(chunks, splits);
+    p.chunks_per_block = cdiv(cdiv(chunks, splits), 4) * 4;
     p.splits = cdiv(chunks, p.chunks_per_block);
     return p;
 }
+
+// Decode kernel (M <= 16, group 128): a block = one column tile x KW wavefronts along K; a K split
+// across blocks only when the tiles alone cannot fill the GPU.
+struct DecodePlan { int v, kw, splits; };
+DecodePlan make_decode_plan(int64_t N, int64_t K) {
+    DecodePlan p;
+    const int Nw = (int)(N / 8), groups = (int)(K / 128);
+    // 128-byte row segments (V = 2) stream measurably faster than 64-byte ones; use them whenever
+    // the tiles alone give every other CU a block, and then do without a second kernel.
+    p.v = (Nw % 2 == 0 && Nw / 32 >= 128) ? 2 : 1;
+    if (g_force_v == 1 || (g_force_v == 2 && Nw % 2 == 0)) p.v = g_force_v;
+    p.kw = (g_force_kw > 0 && p.v == 1) ? g_force_kw : 4;
+    const int ntiles = cdiv(Nw, 16 * p.v);
+    int splits = g_force_splits > 0 ? g_force_splits : (ntiles >= 128 ? 1 : cdiv(200, ntiles));  // measured optimum: ~200 blocks
+    if (splits > groups / p.kw) splits = groups / p.kw;  // at least one group per wavefront
+    if (splits < 1) splits = 1;
+    p.splits = splits;
+    return p;
+}
+
+inline bool decode_path(int64_t M, int64_t group) { return M <= 16 && group == 128; }
 
 template <int V, int MT>
 void launch_awq(const AwqPlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
@@ -304,13 +574,26 @@ void launch_awq(const AwqPlan& p, const uint16_t* x, int64_t ldx, const uint32_t
 
 using namespace llmq;
 
+extern "C" int llmq_awq_force_plan(int v, int splits, int k_waves) {
+    if (v < 0 || v > 2 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
+    g_force_v = v;
+    g_force_splits = splits;
+    g_force_kw = k_waves;
+    return LLMQ_OK;
+}
+
 extern "C" size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     size_t total = 0;
     for (int64_t m0 = 0; m0 < M; m0 += 64) {
         const int64_t mm = M - m0 < 64 ? M - m0 : 64;
-        const AwqPlan p = make_awq_plan(mm, N, K);
-        const size_t need = p.splits > 1 ? (size_t)p.splits * mm * N * sizeof(float) : 0;
+        const AwqPlan p = make_awq_plan(mm, N, K);  // sized for either kernel (the group size is not known here)
+        size_t need = p.splits > 1 ? (size_t)p.splits * mm * N * sizeof(float) : 0;
+        if (mm <= 16 && K % 128 == 0) {
+            const DecodePlan d = make_decode_plan(N, K);
+            const size_t need2 = d.splits > 1 ? (size_t)d.splits * mm * N * sizeof(float) : 0;
+            if (need2 > need) need = need2;
+        }
         if (need > total) total = need;
     }
     return total;
@@ -324,34 +607,49 @@ extern "C" int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight,
     if (!x || !qweight || !scales || !qzeros || !out) return LLMQ_ERR_NULL;
     if (K == 0 || (K % kChunkK) || (N & 7) || group <= 0 || (K % group) || (group % kChunkK) || ldx < K || (ldx & 7))
         return LLMQ_ERR_SHAPE;
-    if (N > 0x7fffffffLL || K > 0x7fffffffLL || M > 0x7fffffffLL) return LLMQ_ERR_SHAPE;
+    if (N > 0x7fffffffLL || K > 0x7fffffffLL || M > 0x7fffffffLL || ldx * 16 > 0x7fffffffLL) return LLMQ_ERR_SHAPE;
     if (!aligned16(x) || !aligned16(scales) || !aligned16(out) || (reinterpret_cast<uintptr_t>(qweight) & 15u) ||
-        (reinterpret_cast<uintptr_t>(qzeros) & 15u))
+        (reinterpret_cast<uintptr_t>(qzeros) & 15u) || (reinterpret_cast<uintptr_t>(workspace) & 15u))
         return LLMQ_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
+    float* ws = (float*)workspace;
+    const uint32_t* qw = (const uint32_t*)qweight;
+    const uint32_t* qz = (const uint32_t*)qzeros;
+    const uint16_t* sc = (const uint16_t*)scales;
+    const uint16_t* bs = (const uint16_t*)bias;
+    const int Ni = (int)N, Ki = (int)K, Gi = (int)group;
     // tokens are processed in slabs of at most 64 rows (4 MFMA token tiles per weight pass)
     for (int64_t m0 = 0; m0 < M; m0 += 64) {
         const int mm = (int)(M - m0 < 64 ? M - m0 : 64);
-        const AwqPlan p = make_awq_plan(mm, N, K);
-        float* ws = (float*)workspace;
-        if (p.splits > 1 && (!ws || workspace_bytes < (size_t)p.splits * mm * N * sizeof(float)))
-            return LLMQ_ERR_WORKSPACE;
         const uint16_t* xs = (const uint16_t*)x + m0 * ldx;
         uint16_t* os = (uint16_t*)out + m0 * N;
-        const uint32_t* qw = (const uint32_t*)qweight;
-        const uint32_t* qz = (const uint32_t*)qzeros;
-        const uint16_t* sc = (const uint16_t*)scales;
-        const uint16_t* bs = (const uint16_t*)bias;
-        const int Ni = (int)N, Ki = (int)K, Gi = (int)group;
-        if (p.v == 2) launch_awq<2, 1>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
-        else if (p.mt == 1) launch_awq<1, 1>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
-        else if (p.mt == 2) launch_awq<1, 2>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
-        else launch_awq<1, 4>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
+        int splits;
+        if (decode_path(mm, group)) {
+            const DecodePlan d = make_decode_plan(N, K);
+            splits = d.splits;
+            if (splits > 1 && (!ws || workspace_bytes < (size_t)splits * mm * N * sizeof(float))) return LLMQ_ERR_WORKSPACE;
+            const dim3 grid(cdiv(Ni / 8, 16 * d.v), splits);
+#define LLMQ_AWQ_DECODE(VV, KWW) \
+    hipLaunchKernelGGL((awq_gemv_kernel<VV, KWW>), grid, dim3(KWW * kWave), 0, st, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, \
+                       Ki)
+            if (d.v == 2) LLMQ_AWQ_DECODE(2, 4);
+            else if (d.kw == 8) LLMQ_AWQ_DECODE(1, 8);
+            else LLMQ_AWQ_DECODE(1, 4);
+#undef LLMQ_AWQ_DECODE
+        } else {
+            const AwqPlan p = make_awq_plan(mm, N, K);
+            splits = p.splits;
+            if (splits > 1 && (!ws || workspace_bytes < (size_t)splits * mm * N * sizeof(float))) return LLMQ_ERR_WORKSPACE;
+            if (p.mt == 1 && p.v == 2) launch_awq<2, 1>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
+            else if (p.mt == 1) launch_awq<1, 1>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
+            else if (p.mt == 2) launch_awq<1, 2>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
+            else launch_awq<1, 4>(p, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, Ki, Gi, st);
+        }
         if (launch_status() != LLMQ_OK) return LLMQ_ERR_LAUNCH;
-        if (p.splits > 1) {
+        if (splits > 1) {
             const int64_t total = (int64_t)mm * N;
             const int blocks = (int)((total + 255) / 256 < 2048 ? (total + 255) / 256 : 2048);
-            hipLaunchKernelGGL(awq_finish_kernel, dim3(blocks), dim3(256), 0, st, ws, p.splits, total, Ni, bs, os);
+            hipLaunchKernelGGL(awq_finish_kernel, dim3(blocks), dim3(256), 0, st, ws, splits, total, Ni, bs, os);
             if (launch_status() != LLMQ_OK) return LLMQ_ERR_LAUNCH;
         }
     }
