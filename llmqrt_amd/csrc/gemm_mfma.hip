@@ -428,7 +428,9 @@ Plan make_plan(int64_t M, int64_t N, int64_t K) {
     }
     // Cost model calibrated on MI355X (microseconds): a CU runs `per_cu` blocks at a time, a block needs
     // t_tile per 64 bytes of K plus a fixed prologue/epilogue cost; blocks execute in rounds over the
-    // 256 CUs.  Split-K adds a second kernel and the round trip of the fp32/int32 partials.
+    // 256 CUs.  The chip is power-limited under MFMA load: with a fraction f of the CUs busy a K tile
+    // takes (0.52 + 0.48 f) of its full-chip time, so a partly filled round is cheaper than a full one.
+    // Split-K adds a second kernel and the round trip of the fp32/int32 partials.
     struct Model { int cfg, per_cu; double t_tile, fixed; };
     static const Model kModels[] = {
         {1, 1, 0.98, 14.5},   // 256x256, 8 waves
@@ -449,9 +451,11 @@ Plan make_plan(int64_t M, int64_t N, int64_t K) {
             const int kps = cdiv(cdiv(K, sp), s.bk) * s.bk;
             const int eff_sp = cdiv(K, kps);
             if (eff_sp != sp) continue;
-            const double rounds = (double)cdiv(tiles * sp, (int64_t)kNumCu * md.per_cu);
-            double t = rounds * (kps / 64.0 * md.t_tile + md.fixed);
-            if (sp > 1) t += 6.0 + (double)M * N * sp * 8.0 / 3.0e6;
+            const int64_t slots = (int64_t)kNumCu * md.per_cu, blocks = tiles * sp;
+            const int64_t full_rounds = blocks / slots, rest = blocks % slots;
+            double t = full_rounds * (kps / 64.0 * md.t_tile + md.fixed);
+            if (rest) t += kps / 64.0 * md.t_tile * (0.52 + 0.48 * (double)rest / slots) + md.fixed;
+            if (sp > 1) t += 5.0 + (double)M * N * sp * 8.0 / 8.0e6;
             if (t < best_t) { best_t = t; best = Plan{md.cfg, sp, kps}; }
         }
     }
