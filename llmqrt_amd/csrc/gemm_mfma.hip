@@ -124,24 +124,33 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     const int st_a = lds_chunk<C::CPR>(ld_row, ld_c);
     const int st_b = C::BM * C::CPR + st_a;
     uint4 ra[2][C::A_LOADS], rb[2][C::B_LOADS];  // two tiles in flight (register staging)
+    // Loads are unconditional (branch-free), so the compiler can count them and wait for exactly the
+    // tile it is about to store while younger loads stay in flight.  A tile index past the end of this
+    // split's K range re-reads the last tile, a chunk past the ragged end of K re-reads chunk 0 of its
+    // row; both are replaced by zeros when the tile is stored to LDS (the main loop always runs an even
+    // number of tiles).
     auto load_tile = [&](int kt, uint4* a_reg, uint4* b_reg) {
-        const int koff = kt * C::BK;
-        // Tiles past the end of this split's K range load zeros (the main loop always runs an even
-        // number of tiles); inside the range a chunk is skipped only in the ragged last tile.
-        const bool ok = kt < ktiles && (KFULL || ld_c * 16 < k_end - k_begin - koff);
+        int koff = max(min(kt, ktiles - 1), 0) * C::BK;
+        if constexpr (!KFULL) koff -= (ld_c * 16 < k_end - k_begin - koff) ? 0 : ld_c * 16;
 #pragma unroll
-        for (int i = 0; i < C::A_LOADS; i++)
-            a_reg[i] = ok ? *reinterpret_cast<const uint4*>(a_base + a_off[i] + koff) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < C::A_LOADS; i++) a_reg[i] = *reinterpret_cast<const uint4*>(a_base + a_off[i] + koff);
 #pragma unroll
-        for (int i = 0; i < C::B_LOADS; i++)
-            b_reg[i] = ok ? *reinterpret_cast<const uint4*>(b_base + b_off[i] + koff) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < C::B_LOADS; i++) b_reg[i] = *reinterpret_cast<const uint4*>(b_base + b_off[i] + koff);
     };
-    auto store_tile = [&](int stage, const uint4* a_reg, const uint4* b_reg) {
+    auto store_tile = [&](int stage, int kt, const uint4* a_reg, const uint4* b_reg) {
         uint4* s = lds + stage * C::STAGE_CHUNKS;
+        const bool ok = kt < ktiles && (KFULL || ld_c * 16 < k_end - k_begin - kt * C::BK);
+        const uint32_t keep = ok ? 0xffffffffu : 0u;
 #pragma unroll
-        for (int i = 0; i < C::A_LOADS; i++) s[st_a + i * ROWS_STEP * C::CPR] = a_reg[i];
+        for (int i = 0; i < C::A_LOADS; i++) {
+            const uint4 v = a_reg[i];
+            s[st_a + i * ROWS_STEP * C::CPR] = make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
+        }
 #pragma unroll
-        for (int i = 0; i < C::B_LOADS; i++) s[st_b + i * ROWS_STEP * C::CPR] = b_reg[i];
+        for (int i = 0; i < C::B_LOADS; i++) {
+            const uint4 v = b_reg[i];
+            s[st_b + i * ROWS_STEP * C::CPR] = make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
+        }
     };
     // Block barrier that orders LDS traffic only: global loads stay in flight across it.
     auto lds_barrier = [] {
@@ -223,10 +232,38 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
         if (kReads > kPairs) __builtin_amdgcn_sched_group_barrier(0x100, kReads - kPairs, 0);
         if (kMfma > kPairs) __builtin_amdgcn_sched_group_barrier(0x008, kMfma - kPairs, 0);
     };
-    // One K tile: sub-steps 0 .. KSUB-2 read the next sub-step of the same stage; the last sub-step
-    // publishes the next tile (registers -> other stage), crosses the barrier and reads that stage's
-    // first sub-step.  `par` is the fragment-buffer parity on entry (compile-time).
-    auto tile_steps = [&](int stage, auto par_c, const uint4* a_reg, const uint4* b_reg) {
+    // Same for the first sub-step of a tile, which also carries the LDS writes of the next tile: reads
+    // first (one per MFMA), then the writes spread over the remaining MFMAs.
+    auto interleave_reads_writes_with_mfma = [] {
+        constexpr int kReads = (C::TM + C::TN) * (C::FP8 ? 2 : 1), kMfma = C::TM * C::TN;
+        constexpr int kWrites = C::A_LOADS + C::B_LOADS;
+        constexpr int kPairs = kReads < kMfma ? kReads : kMfma;
+#pragma unroll
+        for (int n = 0; n < kPairs; n++) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        if (kReads > kPairs) __builtin_amdgcn_sched_group_barrier(0x100, kReads - kPairs, 0);
+        constexpr int kRest = kMfma - kPairs;
+        if constexpr (kRest > 0) {
+            constexpr int kPer = (kWrites + kRest - 1) / kRest;
+#pragma unroll
+            for (int n = 0; n < kRest; n++) {
+#pragma unroll
+                for (int w = 0; w < kPer; w++)
+                    if (n * kPer + w < kWrites) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one DS write
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
+        } else {
+            __builtin_amdgcn_sched_group_barrier(0x200, kWrites, 0);
+        }
+    };
+    // One K tile.  With two or more sub-steps the next tile (registers -> other stage; nobody reads that
+    // stage any more once the previous tile's barrier is passed) is written to LDS under the MFMAs of
+    // sub-step 0; sub-steps 0 .. KSUB-2 read the next sub-step of the same stage; before the last
+    // sub-step the barrier publishes the other stage, whose first sub-step is read under the last MFMAs.
+    // `par` is the fragment-buffer parity on entry (compile-time).
+    auto tile_steps = [&](int stage, auto par_c, int kt_next, const uint4* a_reg, const uint4* b_reg) {
         constexpr int par = decltype(par_c)::value;
         if constexpr (!C::PIPE) {
 #pragma unroll
@@ -234,17 +271,19 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
                 read_frags(stage, ks, fa[0], fb[0]);
                 mfma_step(fa[0], fb[0]);
             }
-            store_tile(stage ^ 1, a_reg, b_reg);
+            store_tile(stage ^ 1, kt_next, a_reg, b_reg);
             lds_barrier();
         } else {
 #pragma unroll
             for (int ks = 0; ks < C::KSUB - 1; ks++) {
                 read_frags(stage, ks + 1, fa[(par + ks + 1) & 1], fb[(par + ks + 1) & 1]);
+                if (ks == 0) store_tile(stage ^ 1, kt_next, a_reg, b_reg);
                 mfma_step(fa[(par + ks) & 1], fb[(par + ks) & 1]);
-                interleave_reads_with_mfma();
+                if (ks == 0) interleave_reads_writes_with_mfma();
+                else interleave_reads_with_mfma();
                 __builtin_amdgcn_sched_barrier(0);
             }
-            store_tile(stage ^ 1, a_reg, b_reg);
+            if constexpr (C::KSUB == 1) store_tile(stage ^ 1, kt_next, a_reg, b_reg);
             lds_barrier();
             read_frags(stage ^ 1, 0, fa[(par + C::KSUB) & 1], fb[(par + C::KSUB) & 1]);
             mfma_step(fa[(par + C::KSUB - 1) & 1], fb[(par + C::KSUB - 1) & 1]);
@@ -258,15 +297,15 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     // compute: an odd tile count is padded with a zero tile -----------------------------------
     load_tile(0, ra[0], rb[0]);
     load_tile(1, ra[1], rb[1]);
-    store_tile(0, ra[0], rb[0]);
+    store_tile(0, 0, ra[0], rb[0]);
     lds_barrier();
     if constexpr (C::PIPE) read_frags(0, 0, fa[0], fb[0]);
 #pragma unroll 1
     for (int kt = 0; kt < ktiles; kt += 2) {
         load_tile(kt + 2, ra[0], rb[0]);
-        tile_steps(0, std::integral_constant<int, 0>{}, ra[1], rb[1]);
+        tile_steps(0, std::integral_constant<int, 0>{}, kt + 1, ra[1], rb[1]);
         load_tile(kt + 3, ra[1], rb[1]);
-        tile_steps(1, std::integral_constant<int, C::KSUB & 1>{}, ra[0], rb[0]);
+        tile_steps(1, std::integral_constant<int, C::KSUB & 1>{}, kt + 2, ra[0], rb[0]);
     }
 
     // ---- epilogue.  The weights feed the MFMA row operand, so D is the transposed tile: a lane holds
