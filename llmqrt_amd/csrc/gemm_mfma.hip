@@ -50,9 +50,10 @@ __device__ __forceinline__ uint16_t to_out(float v, int out_dtype) {
     return out_dtype == LLMQ_BF16 ? Lo<LLMQ_BF16>::from_f32(v) : Lo<LLMQ_F16>::from_f32(v);
 }
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, bool FP8_, int AFMT_ = 0>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, bool FP8_, int AFMT_ = 0, int RS_ = 2>
 struct GemmCfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
+    static constexpr int RS = RS_;                     // K tiles staged in registers: 2, or 1 for fat tiles
     static constexpr bool FP8 = FP8_;
     static constexpr int AFMT = AFMT_;                 // fp8 A format selector: 0 e4m3, 1 e5m2
     static constexpr int NT = WM * WN * kWave;
@@ -67,7 +68,7 @@ struct GemmCfg {
     static constexpr size_t LDS_BYTES = 2u * STAGE_CHUNKS * 16u;
     // Double-buffer the MFMA operand fragments (software pipeline LDS reads under MFMAs).  The fp8
     // fragments are twice as wide; with two wavefronts per SIMD (256 registers each) they do not fit twice.
-    static constexpr bool PIPE = !(FP8 && NT > 256);
+    static constexpr bool PIPE = !(FP8 && NT > 256) && !(RS == 1 && NT > 256);
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be 32-aligned");
     static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "tile must split evenly over threads");
     static_assert(CPR == 4 || CPR == 8, "BK must be 64 or 128");
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     for (int i = 0; i < C::B_LOADS; i++) b_off[i] = min(ld_row + i * ROWS_STEP, N - 1 - n0) * (int)ldb;
     const int st_a = lds_chunk<C::CPR>(ld_row, ld_c);
     const int st_b = C::BM * C::CPR + st_a;
-    uint4 ra[2][C::A_LOADS], rb[2][C::B_LOADS];  // two tiles in flight (register staging)
+    uint4 ra[C::RS][C::A_LOADS], rb[C::RS][C::B_LOADS];  // tiles in flight (register staging)
     // Loads are unconditional (branch-free), so the compiler can count them and wait for exactly the
     // tile it is about to store while younger loads stay in flight.  A tile index past the end of this
     // split's K range re-reads the last tile, a chunk past the ragged end of K re-reads chunk 0 of its
@@ -263,7 +264,7 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     // sub-step 0; sub-steps 0 .. KSUB-2 read the next sub-step of the same stage; before the last
     // sub-step the barrier publishes the other stage, whose first sub-step is read under the last MFMAs.
     // `par` is the fragment-buffer parity on entry (compile-time).
-    auto tile_steps = [&](int stage, auto par_c, int kt_next, const uint4* a_reg, const uint4* b_reg) {
+    auto tile_steps = [&](int stage, auto par_c, int kt_next, uint4* a_reg, uint4* b_reg) {
         constexpr int par = decltype(par_c)::value;
         if constexpr (!C::PIPE) {
 #pragma unroll
@@ -272,18 +273,20 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
                 mfma_step(fa[0], fb[0]);
             }
             store_tile(stage ^ 1, kt_next, a_reg, b_reg);
+            if constexpr (C::RS == 1) load_tile(kt_next + 1, a_reg, b_reg);
             lds_barrier();
         } else {
 #pragma unroll
             for (int ks = 0; ks < C::KSUB - 1; ks++) {
                 read_frags(stage, ks + 1, fa[(par + ks + 1) & 1], fb[(par + ks + 1) & 1]);
-                if (ks == 0) store_tile(stage ^ 1, kt_next, a_reg, b_reg);
+                if (C::RS == 2 && ks == 0) store_tile(stage ^ 1, kt_next, a_reg, b_reg);
                 mfma_step(fa[(par + ks) & 1], fb[(par + ks) & 1]);
-                if (ks == 0) interleave_reads_writes_with_mfma();
+                if (C::RS == 2 && ks == 0) interleave_reads_writes_with_mfma();
                 else interleave_reads_with_mfma();
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (C::KSUB == 1) store_tile(stage ^ 1, kt_next, a_reg, b_reg);
+            if constexpr (C::KSUB == 1 || C::RS == 1) store_tile(stage ^ 1, kt_next, a_reg, b_reg);
+            if constexpr (C::RS == 1) load_tile(kt_next + 1, a_reg, b_reg);  // refill the single register stage
             lds_barrier();
             read_frags(stage ^ 1, 0, fa[(par + C::KSUB) & 1], fb[(par + C::KSUB) & 1]);
             mfma_step(fa[(par + C::KSUB - 1) & 1], fb[(par + C::KSUB - 1) & 1]);
@@ -295,17 +298,32 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     // ---- main loop: tile kt is computed from LDS stage kt & 1 while tile kt+1 sits in registers
     // and tile kt+2 is in flight from global memory.  Two tiles per iteration, no conditional
     // compute: an odd tile count is padded with a zero tile -----------------------------------
-    load_tile(0, ra[0], rb[0]);
-    load_tile(1, ra[1], rb[1]);
-    store_tile(0, 0, ra[0], rb[0]);
-    lds_barrier();
-    if constexpr (C::PIPE) read_frags(0, 0, fa[0], fb[0]);
+    if constexpr (C::RS == 2) {
+        load_tile(0, ra[0], rb[0]);
+        load_tile(1, ra[1], rb[1]);
+        store_tile(0, 0, ra[0], rb[0]);
+        lds_barrier();
+        if constexpr (C::PIPE) read_frags(0, 0, fa[0], fb[0]);
 #pragma unroll 1
-    for (int kt = 0; kt < ktiles; kt += 2) {
-        load_tile(kt + 2, ra[0], rb[0]);
-        tile_steps(0, std::integral_constant<int, 0>{}, kt + 1, ra[1], rb[1]);
-        load_tile(kt + 3, ra[1], rb[1]);
-        tile_steps(1, std::integral_constant<int, C::KSUB & 1>{}, kt + 2, ra[0], rb[0]);
+        for (int kt = 0; kt < ktiles; kt += 2) {
+            load_tile(kt + 2, ra[0], rb[0]);
+            tile_steps(0, std::integral_constant<int, 0>{}, kt + 1, ra[1], rb[1]);
+            load_tile(kt + 3, ra[1], rb[1]);
+            tile_steps(1, std::integral_constant<int, C::KSUB & 1>{}, kt + 2, ra[0], rb[0]);
+        }
+    } else {
+        // fat tiles: one register stage; tile kt+1 is stored late in tile kt and the stage is refilled
+        // with tile kt+2 right away, which then has a whole tile time to arrive
+        load_tile(0, ra[0], rb[0]);
+        store_tile(0, 0, ra[0], rb[0]);
+        load_tile(1, ra[0], rb[0]);
+        lds_barrier();
+        if constexpr (C::PIPE) read_frags(0, 0, fa[0], fb[0]);
+#pragma unroll 1
+        for (int kt = 0; kt < ktiles; kt += 2) {
+            tile_steps(0, std::integral_constant<int, 0>{}, kt + 1, ra[0], rb[0]);
+            tile_steps(1, std::integral_constant<int, C::KSUB & 1>{}, kt + 2, ra[0], rb[0]);
+        }
     }
 
     // ---- epilogue.  The weights feed the MFMA row operand, so D is the transposed tile: a lane holds
@@ -444,6 +462,7 @@ constexpr TileShape kShapes[] = {
     {128, 128, 64},   // 3: 4 waves x (64x64)
     {64, 128, 128},   // 4: 4 waves x (32x64)
     {32, 128, 128},   // 5: 4 waves x (32x32), decode
+    {256, 256, 128},  // 6: 8 waves x (128x64), whole 128-byte lines per row (fp8 prefill)
 };
 constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
 
@@ -532,6 +551,7 @@ int launch_gemm(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, in
         case 2: rc = launch_cfg<GemmCfg<256, 128, 64, 2, 2, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
         case 3: rc = launch_cfg<GemmCfg<128, 128, 64, 2, 2, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
         case 4: rc = launch_cfg<GemmCfg<64, 128, 128, 2, 2, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
+        case 6: rc = launch_cfg<GemmCfg<256, 256, 128, 2, 4, FP8, AFMT, 1>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
         default: rc = launch_cfg<GemmCfg<32, 128, 128, 1, 4, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
     }
     if (rc != LLMQ_OK || p.splits == 1) return rc;
@@ -555,7 +575,9 @@ int gemm_entry(bool fp8, int a_format, const uint8_t* A, int64_t lda, const uint
     if (bias && bias_dtype != LLMQ_BF16 && bias_dtype != LLMQ_F16 && bias_dtype != LLMQ_F32) return LLMQ_ERR_DTYPE;
     if (fp8 && a_format != LLMQ_E4M3 && a_format != LLMQ_E5M2) return LLMQ_ERR_DTYPE;
     if (!aligned16(A) || !aligned16(B)) return LLMQ_ERR_ALIGN;
-    const Plan p = make_plan(M, N, K);
+    Plan p = make_plan(M, N, K);
+    // fp8 fragments are twice as wide: the 8-wave prefill tile runs ~5 % faster with 128-byte K tiles
+    if (fp8 && g_force_cfg < 0 && p.cfg == 1 && p.splits == 1) p.cfg = 6;
     if (p.splits > 1) {
         if (!ws || ws_bytes < (size_t)p.splits * M * N * 4) return LLMQ_ERR_WORKSPACE;
     }
