@@ -269,6 +269,44 @@ def details_layer(dev):
     return out
 
 
+def details_norm_quant(dev):
+    """RMSNorm feeding the per-token int8 quantizer: one fused kernel against the two separate ones."""
+    from llmqrt_amd import _abi, workloads as W
+    L = _abi.lib()
+    stream_obj = torch.cuda.current_stream()
+    stream = stream_obj.cuda_stream
+    out = []
+    K = 3584
+    w = torch.ones(K, dtype=torch.bfloat16, device=dev)
+    for M in (32, 2048, 8192):
+        x = W.activations(M, K, W.seed_for(4, 300 + M % 97)).to(dev)
+        y = torch.empty_like(x)
+        q = torch.empty((M, K), dtype=torch.int8, device=dev)
+        sc = torch.empty(M, dtype=torch.float32, device=dev)
+
+        def fused():
+            return L.llmq_rmsnorm_quant_i8_per_token(x.data_ptr(), 0, M, K, K, w.data_ptr(), 1e-6, None, q.data_ptr(),
+                                                     sc.data_ptr(), 2, None, stream)
+
+        def norm():
+            return L.llmq_rmsnorm(x.data_ptr(), 0, M, K, K, w.data_ptr(), 1e-6, y.data_ptr(), None, stream)
+
+        def quant():
+            return L.llmq_quant_i8_per_token(y.data_ptr(), 0, M, K, K, q.data_ptr(), sc.data_ptr(), 2, stream)
+
+        def two():
+            norm()
+            return quant()
+        assert fused() == 0 and two() == 0
+        tf = batch_time_us([fused], stream_obj, 20)
+        tt = batch_time_us([two], stream_obj, 20)
+        fused_bytes = 3 * M * K + 4 * M + 2 * K
+        out.append({"M": M, "K": K, "fused_us": round(tf, 2), "norm_then_quant_us": round(tt, 2),
+                    "fused_GBs": round(fused_bytes / tf / 1e3, 1),
+                    "pct_hbm_peak": round(100 * fused_bytes / tf / 1e3 / PEAK_HBM_GBS, 2)})
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -400,6 +438,7 @@ def main():
         result["details"]["fp8"] = details_fp8(dev)
         result["details"]["awq_w4a16"] = details_awq(dev)
         result["details"]["layer_stack_w8a8"] = details_layer(dev)
+        result["details"]["rmsnorm_quant_i8"] = details_norm_quant(dev)
 
     print(json.dumps(result))
 

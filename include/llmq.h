@@ -78,6 +78,30 @@ int llmq_quant_fp8_static(const void* x, int x_dtype, int64_t M, int64_t K, int6
 size_t llmq_quant_workspace_bytes(void);
 
 /* ------------------------------------------------------------------------------------
+ * RMSNorm, alone or fused with the per-token quantizer of the Linear that follows it.
+ * Replaces RMSNorm.forward (nn_models/modules/nonlinear/norm.py:10-16), and for the fused
+ * forms also the quantizer call of the next Linear (block.py:68,76 -> linear_sq.py:55-65 /
+ * linear_fp8.py:40-63): the activations make one trip through HBM instead of three.
+ *   h = fp32(x); inv = 1/sqrt(mean_k(h^2) + eps); n = x_dtype(h * inv); y = x_dtype(weight * n)
+ * x: [M, K] bf16/f16 (K % 8 == 0, ldx % 8 == 0, 16-byte aligned); weight: [K] in x_dtype.
+ * y: [M, K] contiguous in x_dtype - required by llmq_rmsnorm, optional (may be NULL) for the
+ * fused forms, which then never write the normalised activations.  q / scale: as for
+ * llmq_quant_i8_per_token / llmq_quant_fp8_per_token applied to y.  inv_rms: optional fp32
+ * [M] that receives inv (parity checks).  Given inv, every output is bit-identical to the
+ * reference; inv itself depends on the summation order of the mean.
+ * ------------------------------------------------------------------------------------ */
+int llmq_rmsnorm(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                 const void* weight, float eps, void* y, float* inv_rms, llmq_stream_t stream);
+int llmq_rmsnorm_quant_i8_per_token(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                    const void* weight, float eps, void* y,
+                                    int8_t* q, void* scale, int scale_dtype,
+                                    float* inv_rms, llmq_stream_t stream);
+int llmq_rmsnorm_quant_fp8_per_token(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                     const void* weight, float eps, void* y,
+                                     uint8_t* q, float* scale,
+                                     float* inv_rms, llmq_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
  * W8A8 int8 GEMM.  Replaces w8a8_int8_linear_bbf16_obf16_per_tensor
  * (csrc/smoothquant/sq_gemm.cu:36-160, bound at csrc/bindings.cpp:10-11) and implements the
  * per-token x per-channel op the reference only declares

@@ -4,6 +4,7 @@ Layout:
   csrc/            HIP kernels + C ABI (include/llmq.h) -> lib/libllmq_gfx950.so
   _abi.py          ctypes loader (no fallback: a missing library raises)
   quantize.py      activation quantizers (reference names)
+  norm.py          RMSNorm, alone or fused with the per-token quantizer
   sq_fp8_kernels   drop-in for runtime.sq_fp8_kernels
   awq_kernels      drop-in for runtime.triton_kernels.awq_kernels
   linear/          quantized Linear modules + registry

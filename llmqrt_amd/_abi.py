@@ -29,6 +29,9 @@ SIGNATURES = {
     "llmq_quant_fp8_per_token": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "llmq_quant_fp8_per_tensor": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
     "llmq_quant_fp8_static": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _int, _vp]),
+    "llmq_rmsnorm": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _f32, _vp, _vp, _vp]),
+    "llmq_rmsnorm_quant_i8_per_token": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _f32, _vp, _vp, _vp, _int, _vp, _vp]),
+    "llmq_rmsnorm_quant_fp8_per_token": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _f32, _vp, _vp, _vp, _vp, _vp]),
     "llmq_quant_workspace_bytes": (_sz, []),
     "llmq_gemm_w8a8": (_int, [_vp, _i64, _vp, _i64, _vp, _vp, _f32, _vp, _vp, _int, _f32, _vp, _int, _i64,
                               _i64, _i64, _i64, _vp, _vp, _sz, _vp]),

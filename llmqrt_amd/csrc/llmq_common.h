@@ -52,6 +52,26 @@ __device__ __forceinline__ float block_max(float v, float* smem) {
     return r;
 }
 
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+// sum over a block of NW wavefronts in a fixed order; every thread gets the same result.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* smem) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+    __syncthreads();
+    if (lane == 0) smem[w] = v;
+    __syncthreads();
+    float r = smem[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) r += smem[i];
+    return r;
+}
+
 inline int launch_status() { return hipGetLastError() == hipSuccess ? LLMQ_OK : LLMQ_ERR_LAUNCH; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

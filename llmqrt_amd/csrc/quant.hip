@@ -183,6 +183,151 @@ __global__ __launch_bounds__(kThreads) void absmax_partials_kernel(
     if (threadIdx.x == 0) partials[blockIdx.x] = amax;
 }
 
+// ---- RMSNorm fused with the per-token quantizer --------------------------------------------
+// The reference normalises (nn_models/modules/nonlinear/norm.py:10-16) and then quantizes the result in
+// the first Linear of the block (nn_models/modules/nonlinear/block.py:68,76 -> linear_sq.py:55-65 /
+// linear_fp8.py:40-63): two round trips of the activations through HBM.  Here a row is read once, kept
+// in registers, normalised, (optionally) written back as y, and quantized:
+//   h = fp32(x);  inv = 1 / sqrt(mean(h^2) + eps);  n = round_dt(h * inv);  y = round_dt(w * n)
+//   then exactly the per-token quantizer above on y.
+// Everything after `inv` is bit-identical to the reference evaluated with the same inv; inv itself
+// depends on the summation order of mean() (here: per-thread FMA chain, wavefront butterfly, then the
+// wavefronts in order) and can differ from another order in the last bits.
+template <int DT>
+__device__ __forceinline__ float sumsq8(uint4 r, float acc) {
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float a = Lo<DT>::to_f32((uint16_t)(w[i] & 0xffffu)), b = Lo<DT>::to_f32((uint16_t)(w[i] >> 16));
+        acc = fmaf(a, a, acc);
+        acc = fmaf(b, b, acc);
+    }
+    return acc;
+}
+
+template <int DT>
+__device__ __forceinline__ uint4 norm8(uint4 r, uint4 wv, float inv) {
+    const uint32_t x[4] = {r.x, r.y, r.z, r.w}, w[4] = {wv.x, wv.y, wv.z, wv.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        // The reference rounds the product to fp32 and then to the activation dtype.  Keep the fp32 product
+        // opaque so that the compiler cannot fuse multiply and narrowing into one mixed-precision
+        // instruction, which rounds once and lands on the other side of a tie now and then.
+        float p0 = Lo<DT>::to_f32((uint16_t)(x[i] & 0xffffu)) * inv;
+        float p1 = Lo<DT>::to_f32((uint16_t)(x[i] >> 16)) * inv;
+        asm volatile("" : "+v"(p0), "+v"(p1));
+        const float n0 = Lo<DT>::round(p0), n1 = Lo<DT>::round(p1);
+        const uint16_t y0 = Lo<DT>::from_f32(Lo<DT>::to_f32((uint16_t)(w[i] & 0xffffu)) * n0);
+        const uint16_t y1 = Lo<DT>::from_f32(Lo<DT>::to_f32((uint16_t)(w[i] >> 16)) * n1);
+        o[i] = (uint32_t)y0 | ((uint32_t)y1 << 16);
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// QMODE: -1 = no quantizer (plain RMSNorm), MODE_I8, MODE_F8.
+template <int DT, int QMODE, int NC>
+__global__ __launch_bounds__(kThreads) void rmsnorm_quant_rows_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, int64_t K, const uint16_t* __restrict__ weight, float eps,
+    uint16_t* __restrict__ y, uint8_t* __restrict__ q, void* __restrict__ scale_out, int scale_dtype,
+    float* __restrict__ inv_out) {
+    __shared__ float smem[kNW];
+    constexpr int QM = QMODE < 0 ? MODE_I8 : QMODE;
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int nchunk = (int)(K >> 3);
+    const uint4* xr = reinterpret_cast<const uint4*>(x + row * ldx);
+    const uint4* wr = reinterpret_cast<const uint4*>(weight);
+    uint4* yr = y ? reinterpret_cast<uint4*>(y + row * K) : nullptr;
+    uint2* qr = reinterpret_cast<uint2*>(q + row * K);
+
+    uint4 cache[NC > 0 ? NC : 1];
+    float ss = 0.f;
+    if (NC > 0) {
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+            const int i = tid + c * kThreads;
+            cache[c] = (i < nchunk) ? xr[i] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < NC; c++) ss = sumsq8<DT>(cache[c], ss);
+    } else {
+        for (int i = tid; i < nchunk; i += kThreads) ss = sumsq8<DT>(xr[i], ss);
+    }
+    ss = block_sum<kNW>(ss, smem);
+    const float inv = 1.0f / sqrtf(ss / (float)K + eps);
+    if (inv_out && tid == 0) inv_out[row] = inv;
+
+    float amax = 0.f;
+    if (NC > 0) {
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+            const int i = tid + c * kThreads;
+            if (i < nchunk) {
+                cache[c] = norm8<DT>(cache[c], wr[i], inv);
+                if (yr) yr[i] = cache[c];
+                amax = fmaxf(amax, absmax8(cache[c], DT == LLMQ_BF16));
+            }
+        }
+    } else {
+        for (int i = tid; i < nchunk; i += kThreads) {
+            const uint4 v = norm8<DT>(xr[i], wr[i], inv);
+            if (yr) yr[i] = v;
+            amax = fmaxf(amax, absmax8(v, DT == LLMQ_BF16));
+        }
+    }
+    if (QMODE < 0) return;
+    amax = block_max<kNW>(amax, smem);
+    const float s = scale_from_amax<DT, QM>(amax);
+    if (tid == 0) {
+        if (scale_dtype == LLMQ_F32) ((float*)scale_out)[row] = s;
+        else ((uint16_t*)scale_out)[row] = Lo<DT>::from_f32(s);
+    }
+    const float inv_s = 1.0f / s;
+    if (NC > 0) {
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+            const int i = tid + c * kThreads;
+            if (i < nchunk) qr[i] = quant8<DT, QM, Q_DT>(cache[c], s, inv_s);
+        }
+    } else {
+        for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, QM, Q_DT>(norm8<DT>(xr[i], wr[i], inv), s, inv_s);
+    }
+}
+
+template <int DT, int QMODE>
+int launch_norm(const void* x, int64_t M, int64_t K, int64_t ldx, const void* weight, float eps, void* y, void* q,
+                void* scale, int scale_dtype, float* inv_out, hipStream_t st) {
+    const dim3 grid((unsigned)M), block(kThreads);
+    const int64_t per_thread = ((K >> 3) + kThreads - 1) / kThreads;
+#define LLMQ_LAUNCH_NC(NC)                                                                                      \
+    hipLaunchKernelGGL((rmsnorm_quant_rows_kernel<DT, QMODE, NC>), grid, block, 0, st, (const uint16_t*)x, ldx, K, \
+                       (const uint16_t*)weight, eps, (uint16_t*)y, (uint8_t*)q, scale, scale_dtype, inv_out)
+    if (per_thread <= 1) LLMQ_LAUNCH_NC(1);
+    else if (per_thread <= 2) LLMQ_LAUNCH_NC(2);
+    else if (per_thread <= 4) LLMQ_LAUNCH_NC(4);
+    else if (per_thread <= 10) LLMQ_LAUNCH_NC(10);
+    else LLMQ_LAUNCH_NC(0);
+#undef LLMQ_LAUNCH_NC
+    return launch_status();
+}
+
+template <int QMODE>
+int rmsnorm_entry(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, const void* weight, float eps,
+                  void* y, void* q, void* scale, int scale_dtype, float* inv_out, hipStream_t st) {
+    if (x_dtype != LLMQ_BF16 && x_dtype != LLMQ_F16) return LLMQ_ERR_DTYPE;
+    if (M < 0 || K < 0 || ldx < K || (K & 7) || (ldx & 7) || M > 0x7fffffffLL) return LLMQ_ERR_SHAPE;
+    if (M == 0) return LLMQ_OK;
+    if (K == 0) return LLMQ_ERR_SHAPE;
+    if (!x || !weight || (QMODE < 0 ? !y : (!q || !scale))) return LLMQ_ERR_NULL;
+    if (QMODE >= 0 && scale_dtype != x_dtype && scale_dtype != LLMQ_F32) return LLMQ_ERR_DTYPE;
+    if (!aligned16(x) || !aligned16(weight) || (y && !aligned16(y)) || (q && (reinterpret_cast<uintptr_t>(q) & 7u)))
+        return LLMQ_ERR_ALIGN;
+    if (x_dtype == LLMQ_BF16)
+        return launch_norm<LLMQ_BF16, QMODE>(x, M, K, ldx, weight, eps, y, q, scale, scale_dtype, inv_out, st);
+    return launch_norm<LLMQ_F16, QMODE>(x, M, K, ldx, weight, eps, y, q, scale, scale_dtype, inv_out, st);
+}
+
 int check_common(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, const void* q) {
     if (!x || !q) return (M == 0 || K == 0) ? LLMQ_OK : LLMQ_ERR_NULL;
     if (x_dtype != LLMQ_BF16 && x_dtype != LLMQ_F16) return LLMQ_ERR_DTYPE;
@@ -298,4 +443,24 @@ extern "C" int llmq_quant_fp8_static(const void* x, int x_dtype, int64_t M, int6
     if (!scale) return LLMQ_ERR_NULL;
     return dispatch_rows<MODE_F8, SCALE_STATIC>(x, x_dtype, M, K, ldx, q, nullptr, LLMQ_F32, scale, 1,
                                                 scale_is_f32_tensor ? 1 : 0, (hipStream_t)stream);
+}
+
+extern "C" int llmq_rmsnorm(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, const void* weight,
+                            float eps, void* y, float* inv_rms, llmq_stream_t stream) {
+    return rmsnorm_entry<-1>(x, x_dtype, M, K, ldx, weight, eps, y, nullptr, nullptr, LLMQ_F32, inv_rms,
+                             (hipStream_t)stream);
+}
+
+extern "C" int llmq_rmsnorm_quant_i8_per_token(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                               const void* weight, float eps, void* y, int8_t* q, void* scale,
+                                               int scale_dtype, float* inv_rms, llmq_stream_t stream) {
+    return rmsnorm_entry<MODE_I8>(x, x_dtype, M, K, ldx, weight, eps, y, q, scale, scale_dtype, inv_rms,
+                                  (hipStream_t)stream);
+}
+
+extern "C" int llmq_rmsnorm_quant_fp8_per_token(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                                const void* weight, float eps, void* y, uint8_t* q, float* scale,
+                                                float* inv_rms, llmq_stream_t stream) {
+    return rmsnorm_entry<MODE_F8>(x, x_dtype, M, K, ldx, weight, eps, y, q, scale, LLMQ_F32, inv_rms,
+                                  (hipStream_t)stream);
 }

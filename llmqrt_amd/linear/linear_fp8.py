@@ -89,6 +89,15 @@ class FP8DynamicLinear(_FP8LinearBase):
                                                    x_scale.view(-1, 1), self.weight_scale.to(torch.float32).t(), True)
         return output.view(*x_shape[:-1], -1)
 
+    @torch.no_grad()
+    def forward_quantized(self, qinput, x_scale):
+        """Per-channel forward for activations already quantized per token (e4m3fn qinput, fp32 scales
+        [.., 1]), e.g. by the fused RMSNorm + quantizer kernel; no counterpart in the reference."""
+        assert not self.per_tensor, "pre-quantized activations carry per-token scales"
+        output = cutlass_f8f8bf16_rowwise_sm89(qinput.reshape(-1, qinput.shape[-1]), self._qweight_t(), self.bias,
+                                               x_scale.reshape(-1, 1), self.weight_scale.to(torch.float32).t(), True)
+        return output.view(*qinput.shape[:-1], -1)
+
 
 class FP8StaticLinear(_FP8LinearBase):
     def __init__(self, in_features, out_features, bias, dev="cuda:0", dtype=torch.bfloat16,

@@ -114,6 +114,15 @@ class SqW8A8BBF16OBF16PerChannel(LinearBase):
                                                      input_scale, self.weight_scale)
         return y.view(*x_shape[:-1], -1)
 
+    @torch.no_grad()
+    def forward_quantized(self, qx, input_scale, out_dtype):
+        """Same as forward for activations that are already quantized per token (int8 qx, fp32 scales
+        [.., 1]), e.g. by the fused RMSNorm + quantizer kernel; no counterpart in the reference."""
+        q2 = qx.reshape(-1, qx.shape[-1])
+        y = w8a8_int8_linear_bbf16_obf16_per_channel(q2, self.qweight.t(), self._bias_or_zeros(out_dtype, qx.device),
+                                                     input_scale.reshape(-1, 1), self.weight_scale)
+        return y.view(*qx.shape[:-1], -1)
+
     @classmethod
     def from_linear(cls, module: torch.nn.Linear, w_bit, group_size, init_only=True, dtype=torch.float16,
                     per_tensor=False):

@@ -115,3 +115,20 @@ def e4m3_decode_table():
 
 def e4m3_encode(values):
     return np.array([lib().orc_e4m3_encode(float(v)) for v in values], np.uint8)
+
+
+def rmsnorm_given_inv(x: torch.Tensor, weight: torch.Tensor, inv: torch.Tensor) -> torch.Tensor:
+    M, K = x.shape
+    xb, wb = _u16(x), _u16(weight)
+    iv = np.ascontiguousarray(inv.reshape(M).to(torch.float32).numpy())
+    y = np.empty((M, K), np.uint16)
+    lib().orc_rmsnorm_given_inv(_p(xb), _p(wb), _p(iv), _dt(x), ctypes.c_long(M), ctypes.c_long(K), _p(y))
+    return torch.from_numpy(y.view(np.int16)).view(x.dtype)
+
+
+def inv_rms_f64(x: torch.Tensor, eps: float) -> torch.Tensor:
+    M, K = x.shape
+    xb = _u16(x)
+    out = np.empty((M,), np.float64)
+    lib().orc_inv_rms_f64(_p(xb), _dt(x), ctypes.c_long(M), ctypes.c_long(K), ctypes.c_double(eps), _p(out))
+    return torch.from_numpy(out)

@@ -187,3 +187,26 @@ void orc_awq_gemm(const uint16_t* x, const int32_t* qweight, const int32_t* qzer
             out[m * N + n] = f32_to_f16((float)s);
         }
 }
+
+/* ---- RMSNorm given the reciprocal RMS (nn_models/modules/nonlinear/norm.py:14-16):
+ * y = round_dt(w * round_dt(fp32(x) * inv)), scalar loops. */
+void orc_rmsnorm_given_inv(const uint16_t* x, const uint16_t* w, const float* inv, int dt, long M, long K,
+                           uint16_t* y) {
+    for (long m = 0; m < M; m++)
+        for (long k = 0; k < K; k++) {
+            const float n = lo_to_f32(f32_to_lo(lo_to_f32(x[m * K + k], dt) * inv[m], dt), dt);
+            y[m * K + k] = f32_to_lo(lo_to_f32(w[k], dt) * n, dt);
+        }
+}
+
+/* Reciprocal RMS with the mean accumulated in double (the value every fp32 summation order approximates). */
+void orc_inv_rms_f64(const uint16_t* x, int dt, long M, long K, double eps, double* inv) {
+    for (long m = 0; m < M; m++) {
+        double ss = 0.0;
+        for (long k = 0; k < K; k++) {
+            const double h = (double)lo_to_f32(x[m * K + k], dt);
+            ss += h * h;
+        }
+        inv[m] = 1.0 / sqrt(ss / (double)K + eps);
+    }
+}

@@ -121,6 +121,22 @@ def w8a8_linear_naive(qx, a_scale, qw_nk, w_scale, bias, out_dtype):
 # FP8 (OCP e4m3fn)
 # --------------------------------------------------------------------------------------
 @torch.no_grad()
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float):
+    """RMSNorm.forward, nn_models/modules/nonlinear/norm.py:10-16, line by line.  -> (y in x.dtype, inv fp32 [.., 1]).
+
+    The mean is whatever order torch's CPU reduction uses: `inv` is pinned only to a few fp32 ulps (see
+    rmsnorm_given_inv for the part that is pinned bit for bit)."""
+    h = x.to(torch.float32)
+    variance = h.pow(2).mean(-1, keepdim=True)
+    inv = torch.rsqrt(variance + eps)
+    return weight * (h * inv).to(x.dtype), inv
+
+
+def rmsnorm_given_inv(x: torch.Tensor, weight: torch.Tensor, inv: torch.Tensor) -> torch.Tensor:
+    """Lines 14-16 of the same function with the reciprocal RMS supplied: y = weight * (fp32(x) * inv).to(dtype)."""
+    return weight * (x.to(torch.float32) * inv.to(torch.float32).reshape(*x.shape[:-1], 1)).to(x.dtype)
+
+
 def fp8_per_token_quantize(t: torch.Tensor):
     """nn_models/modules/linear/linear_fp8.py:40-63: scale = clamp(amax, 1e-12) / 448 in
     t.dtype, q = e4m3fn(clamp(t / scale, -448, 448)), scale returned as fp32 [.., 1]."""

@@ -140,3 +140,19 @@ def test_workload_shapes_and_byte_counts():
     assert W.gemm_ops(2048, 4608, 3584) == 67645734912
     assert W.awq_gemm_bytes(1, 4608, 3584) == 8596480                    # 8.60 MB
     assert W.w8a8_gemm_bytes(16, 4864, 896) == 4547648                   # 4.55 MB
+
+
+def test_rmsnorm_argument_validation_needs_no_gpu():
+    from llmqrt_amd import _abi
+    L = _abi.lib()
+    ok_ptr = 0x1000
+    # null weight / output, bad dtype, K not a multiple of 8, misaligned input
+    assert L.llmq_rmsnorm(ok_ptr, 0, 4, 64, 64, None, 1e-6, ok_ptr, None, None) == -1
+    assert L.llmq_rmsnorm(ok_ptr, 0, 4, 64, 64, ok_ptr, 1e-6, None, None, None) == -1
+    assert L.llmq_rmsnorm(ok_ptr, 2, 4, 64, 64, ok_ptr, 1e-6, ok_ptr, None, None) == -2
+    assert L.llmq_rmsnorm(ok_ptr, 0, 4, 60, 64, ok_ptr, 1e-6, ok_ptr, None, None) == -3
+    assert L.llmq_rmsnorm(ok_ptr + 2, 0, 4, 64, 64, ok_ptr, 1e-6, ok_ptr, None, None) == -6
+    assert L.llmq_rmsnorm(ok_ptr, 0, 0, 64, 64, ok_ptr, 1e-6, ok_ptr, None, None) == 0
+    assert L.llmq_rmsnorm_quant_i8_per_token(ok_ptr, 0, 4, 64, 64, ok_ptr, 1e-6, None, None, ok_ptr, 0, None, None) == -1
+    assert L.llmq_rmsnorm_quant_i8_per_token(ok_ptr, 0, 4, 64, 64, ok_ptr, 1e-6, None, ok_ptr, ok_ptr, 1, None, None) == -2
+    assert L.llmq_rmsnorm_quant_fp8_per_token(ok_ptr, 1, 4, 64, 32, ok_ptr, 1e-6, None, ok_ptr, ok_ptr, None, None) == -3

@@ -219,3 +219,51 @@ def test_awq_dequant_torch_vs_scalar_c_and_closed_form():
     x = W.activations(3, 256, 4, dtype=torch.float16, outliers=False)
     y1, y2 = R.awq_gemm(x, qw, qz, s, 64), C.awq_gemm(x, qw, qz, s, 64)
     assert (y1.float() - y2.float()).abs().max() <= 2e-3 * y1.float().abs().max()
+
+
+# ---- RMSNorm ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rmsnorm_closed_forms(dtype):
+    eps = 1e-6
+    # a constant row c has RMS |c|: inv = 1/sqrt(c^2 + eps), y = w * round(c * inv)
+    c = 3.0
+    x = torch.full((2, 64), c, dtype=dtype)
+    w = torch.linspace(-2, 2, 64).to(dtype)
+    y, inv = R.rmsnorm(x, w, eps)
+    assert torch.allclose(inv, torch.full((2, 1), 1.0 / math.sqrt(c * c + eps)), rtol=3e-7, atol=0)
+    n = torch.tensor(c * (1.0 / math.sqrt(c * c + eps))).to(dtype)      # rounds to exactly 1.0
+    assert float(n) == 1.0
+    assert torch.equal(y, w.expand(2, 64))
+    # a single spike of height a in K zeros: mean = a^2 / K
+    x = torch.zeros(1, 256, dtype=dtype)
+    x[0, 17] = -8.0
+    y, inv = R.rmsnorm(x, torch.ones(256, dtype=dtype), 0.0)
+    assert float(inv) == pytest.approx(math.sqrt(256) / 8.0, rel=3e-7)
+    assert float(y[0, 17]) == -16.0 and float(y.abs().sum()) == 16.0
+    # an all-zero row: inv = 1/sqrt(eps), output exactly zero
+    y, inv = R.rmsnorm(torch.zeros(1, 64, dtype=dtype), w, eps)
+    assert float(inv) == pytest.approx(1000.0, rel=3e-7) and not y.any()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K", [(5, 896), (3, 3584), (2, 8)])
+def test_rmsnorm_torch_vs_scalar_c_and_f64(M, K, dtype):
+    eps = 1e-6
+    x = _acts(M, K, 900 + M + K, dtype)
+    g = torch.Generator().manual_seed(K)
+    w = (1.0 + 0.1 * torch.randn(K, generator=g)).to(dtype)
+    y, inv = R.rmsnorm(x, w, eps)
+    # the reciprocal RMS agrees with a double-precision evaluation to a few fp32 ulps ...
+    inv64 = C.inv_rms_f64(x, eps)
+    assert torch.allclose(inv.view(-1).double(), inv64, rtol=5e-7, atol=0)
+    # ... and everything after it is pinned bit for bit by the independent scalar implementation
+    assert torch.equal(R.rmsnorm_given_inv(x, w, inv).view(torch.int16), y.view(torch.int16))
+    assert torch.equal(C.rmsnorm_given_inv(x, w, inv).view(torch.int16), y.view(torch.int16))
+    # against exact arithmetic the result is within the two roundings of the formula
+    exact = w.double() * (x.double() * inv64.view(M, 1))
+    ulp = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+    assert ((y.double() - exact).abs() <= 2.5 * ulp * exact.abs() + 1e-30).all()
+    # scale invariance: normalising 2x gives the same result up to eps
+    y2, _ = R.rmsnorm((x.float() * 2).to(dtype), w, 0.0)
+    y0, _ = R.rmsnorm(x, w, 0.0)
+    assert (y2.float() - y0.float()).abs().max() <= 2 * ulp * y0.float().abs().max()
