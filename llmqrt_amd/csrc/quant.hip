@@ -29,23 +29,17 @@ __device__ __forceinline__ float scale_from_amax(float amax) {
     return Lo<DT>::round(fmaxf(amax, fl) / QP<MODE>::qmax);
 }
 
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ float absmax8(uint4 r, int dt_is_bf16) {
-    // |x| of 8 packed 16-bit floats: clear the sign bits, compare as fp32
-    const uint32_t w[4] = {r.x & 0x7fff7fffu, r.y & 0x7fff7fffu, r.z & 0x7fff7fffu, r.w & 0x7fff7fffu};
-    float m = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        float a, b;
-        if (dt_is_bf16) {
-            a = __uint_as_float(w[i] << 16);
-            b = __uint_as_float(w[i] & 0xffff0000u);
-        } else {
-            a = Lo<LLMQ_F16>::to_f32((uint16_t)(w[i] & 0xffffu));
-            b = Lo<LLMQ_F16>::to_f32((uint16_t)(w[i] >> 16));
-        }
-        m = fmaxf(m, fmaxf(a, b));
-    }
-    return m;
+    // |x| of 8 packed 16-bit floats.  With the sign bits cleared the bit patterns of bf16 / fp16 values
+    // order like the values themselves, so the maximum is taken on packed unsigned 16-bit integers
+    // (two elements per instruction) and only the winner is widened to fp32.
+    const u16x2 a = __builtin_bit_cast(u16x2, r.x & 0x7fff7fffu), b = __builtin_bit_cast(u16x2, r.y & 0x7fff7fffu);
+    const u16x2 c = __builtin_bit_cast(u16x2, r.z & 0x7fff7fffu), d = __builtin_bit_cast(u16x2, r.w & 0x7fff7fffu);
+    const u16x2 m = __builtin_elementwise_max(__builtin_elementwise_max(a, b), __builtin_elementwise_max(c, d));
+    const uint16_t top = m[0] > m[1] ? m[0] : m[1];
+    return dt_is_bf16 ? __uint_as_float((uint32_t)top << 16) : Lo<LLMQ_F16>::to_f32(top);
 }
 
 // Quotient rounded to the activation dtype.  bf16: x * (1/s) rounds to the same bf16 value
