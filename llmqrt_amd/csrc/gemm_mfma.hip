@@ -334,6 +334,65 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     const float alpha = ep.alpha * (ep.alpha_dev ? *ep.alpha_dev : 1.0f);
     const bool out_vec = ((ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(out) & 15u) == 0);
     const bool raw_vec = (N & 3) == 0;
+
+    // Fast path (block-uniform): interior tile, fused epilogue, vector stores.  No per-element dtype
+    // switches or bounds checks: ~5 VALU operations per output instead of several times that.
+    if (!split && !acc_dump && out_vec && m0 + C::BM <= M && n0 + C::BN <= N &&
+        (reinterpret_cast<uintptr_t>(ep.w_scale) & 15u) == 0) {
+        auto fast = [&](auto out_dt_c) {
+            constexpr int ODT = decltype(out_dt_c)::value;
+#pragma unroll
+            for (int j = 0; j < C::TN; j++) {
+                const int nb = n0 + wn * C::WTN + j * 32;
+                float sw[16], bb[16];
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int n = nb + 8 * g + 4 * khalf;
+                    if (ep.w_scale) {
+                        const float4 v = *reinterpret_cast<const float4*>(ep.w_scale + n);
+                        sw[4 * g] = v.x, sw[4 * g + 1] = v.y, sw[4 * g + 2] = v.z, sw[4 * g + 3] = v.w;
+                    } else {
+                        sw[4 * g] = sw[4 * g + 1] = sw[4 * g + 2] = sw[4 * g + 3] = 1.f;
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        bb[4 * g + e] = ep.bias ? ep.beta * load_as_f32(ep.bias, ep.bias_dtype, n + e) : 0.f;
+                }
+#pragma unroll
+                for (int i = 0; i < C::TM; i++) {
+                    const int m = m0 + wm * C::WTM + i * 32 + l32;
+                    const float sa = ep.a_scale ? ep.a_scale[m] : 1.f;
+                    uint32_t pk[4][2];
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        uint16_t h[4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const auto av = acc[i][j][4 * g + e];
+                            h[e] = Lo<ODT>::from_f32(epi_value((float)av, sa, sw[4 * g + e], alpha, bb[4 * g + e]));
+                        }
+                        pk[g][0] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+                        pk[g][1] = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+                    }
+                    uint16_t* orow = reinterpret_cast<uint16_t*>(out) + (int64_t)m * ldo;
+#pragma unroll
+                    for (int g = 0; g < 2; g++) {
+#pragma unroll
+                        for (int x = 0; x < 2; x++) {
+                            const auto sw2 = __builtin_amdgcn_permlane32_swap(pk[g][x], pk[g + 2][x], false, false);
+                            pk[g][x] = sw2[0];
+                            pk[g + 2][x] = sw2[1];
+                        }
+                        *reinterpret_cast<uint4*>(orow + nb + 16 * khalf + 8 * g) =
+                            make_uint4(pk[g][0], pk[g][1], pk[g + 2][0], pk[g + 2][1]);
+                    }
+                }
+            }
+        };
+        if (ep.out_dtype == LLMQ_BF16) fast(std::integral_constant<int, LLMQ_BF16>{});
+        else fast(std::integral_constant<int, LLMQ_F16>{});
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < C::TN; j++) {
         const int nb = n0 + wn * C::WTN + j * 32;  // first channel of this 32-wide MFMA tile (wave-uniform)
