@@ -235,3 +235,46 @@ def test_fp8_rejects_bad_inputs(cuda):
         cutlass_f8f8bf16_tensorwise_sm89(a, b.t(), None, 1.0, 1.0, "float32")    # unsupported out dtype
     with pytest.raises(RuntimeError):
         cutlass_f8f8bf16_tensorwise_sm89(a, b.t(), torch.zeros(8, dtype=torch.float16, device=cuda), 1.0, 1.0, "bfloat16")
+
+
+# ---- interior-tile fast epilogue ------------------------------------------------------------------
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_fast_epilogue_is_bit_identical_to_the_general_one(cuda, force_plan, out_dtype):
+    """Tiles that lie wholly inside the output take a block-uniform fast epilogue (no accumulator dump, no
+    split).  For every tile configuration its output must equal, bit for bit, what the general epilogue
+    writes for the same problem (selected here by asking for the accumulator dump), and the oracle's."""
+    from llmqrt_amd.sq_fp8_kernels import (cutlass_f8f8bf16_rowwise_sm89, cutlass_f8f8bf16_tensorwise_sm89,
+                                           w8a8_int8_linear_bbf16_obf16_per_channel,
+                                           w8a8_int8_linear_bbf16_obf16_per_tensor)
+    M, N, K = 512, 768, 320   # interior tiles for every configuration; odd K-tile count for BK = 64
+    qx, sx, qw, sw, bias = _int8_problem(M, N, K, 31)
+    bias = bias.to(out_dtype)
+    acc_ref = R.int8_gemm_exact(qx, qw)
+    xq, xs, wq, ws, bias8 = _fp8_problem(M, N, K, 33)
+    for cfg in range(_num_cfgs()):
+        force_plan(cfg, 1)
+        dump = torch.empty((M, N), dtype=torch.int32, device=cuda)
+        args = (qx.to(cuda), qw.to(cuda).t(), bias.to(cuda), sx.to(cuda), sw.to(cuda))
+        if out_dtype == torch.bfloat16:
+            fast = w8a8_int8_linear_bbf16_obf16_per_channel(*args)
+            general = w8a8_int8_linear_bbf16_obf16_per_channel(*args, _acc_dump=dump)
+            y_ref = R.w8a8_epilogue_per_token_per_channel(acc_ref, sx, sw, bias, out_dtype)
+        else:
+            a2 = (qx.to(cuda), qw.to(cuda).t(), bias.to(cuda), 0.0125, 0.5)
+            fast = w8a8_int8_linear_bbf16_obf16_per_tensor(*a2)
+            general = w8a8_int8_linear_bbf16_obf16_per_tensor(*a2, _acc_dump=dump)
+            y_ref = R.w8a8_epilogue_per_tensor(acc_ref, bias, 0.0125, 0.5, out_dtype)
+        assert fast.dtype == out_dtype
+        assert torch.equal(fast.view(torch.int16), general.view(torch.int16)), f"int8 cfg {cfg}"
+        assert torch.equal(dump.cpu(), acc_ref)
+        assert rel_err(fast, y_ref) <= REL_TOL, f"int8 cfg {cfg}"
+        dump8 = torch.empty((M, N), dtype=torch.float32, device=cuda)
+        if out_dtype == torch.bfloat16:
+            a8 = (xq.to(cuda), wq.to(cuda).t(), bias8.to(cuda), xs.to(cuda), ws.to(cuda).view(1, -1), True)
+            fast8 = cutlass_f8f8bf16_rowwise_sm89(*a8)
+            general8 = cutlass_f8f8bf16_rowwise_sm89(*a8, _acc_dump=dump8)
+        else:
+            a8 = (xq.to(cuda), wq.to(cuda).t(), bias8.to(out_dtype).to(cuda), 0.75, 1.0, "float16")
+            fast8 = cutlass_f8f8bf16_tensorwise_sm89(*a8)
+            general8 = cutlass_f8f8bf16_tensorwise_sm89(*a8, _acc_dump=dump8)
+        assert torch.equal(fast8.view(torch.int16), general8.view(torch.int16)), f"fp8 cfg {cfg}"
