@@ -275,7 +275,7 @@ template <int V, int KW>
 __global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, const uint32_t* __restrict__ qw,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qz, const uint16_t* __restrict__ bias,
-    uint16_t* __restrict__ out, float* __restrict__ partials, int M, int N, int K) {
+    uint16_t* __restrict__ out, float* __restrict__ partials, int M_total, int N, int K, int slabs) {
     typedef typename WordVec<V>::type wvec;
     constexpr int G = 128, RING = G / kChunkK, NACC = V * 8;
     __shared__ float4 red[(KW / 2) * NACC * kWave];
@@ -284,14 +284,20 @@ __global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // scalar: keeps the loop bounds uniform
     const int li = lane & 15, kb = lane >> 4;
     const int Nw = N >> 3;
-    // Column tile of this block.  Consecutive block ids are dealt round-robin to the 8 XCDs; give each
-    // XCD a contiguous range of tiles instead, so that the two 64-byte halves of a cache line (adjacent
-    // tiles when V == 1) are fetched through the same L2.
-    int tile = blockIdx.x;
+    // Column tile and token slab of this block.  Consecutive block ids are dealt round-robin to the 8
+    // XCDs; give each XCD a contiguous range of (tile, slab) pairs instead, so that the two 64-byte halves
+    // of a cache line (adjacent tiles when V == 1) and the up to 4 token slabs of 16 rows that stream the
+    // same weights are served by the same L2 at about the same time (HBM sees the weights once).
+    int seq = blockIdx.x;
     {
-        const int nb = gridDim.x, q = nb / 8, r = nb % 8, xcd = tile % 8, local = tile / 8;
-        tile = xcd < r ? xcd * (q + 1) + local : r * (q + 1) + (xcd - r) * q + local;
+        const int nb = gridDim.x, q = nb / 8, r = nb % 8, xcd = seq % 8, local = seq / 8;
+        seq = xcd < r ? xcd * (q + 1) + local : r * (q + 1) + (xcd - r) * q + local;
     }
+    const int tile = seq / slabs, slab = seq - tile * slabs;
+    const int M = min(16, M_total - 16 * slab);  // tokens of this slab
+    x += (int64_t)(16 * slab) * ldx;
+    out += (int64_t)(16 * slab) * N;
+    partials += (int64_t)(16 * slab) * N;
     const int cw = tile * (16 * V) + V * li;  // first word column of this lane
     const bool col_ok = cw < Nw;
     const int cwc = col_ok ? cw : 0;
@@ -449,7 +455,7 @@ __global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
         for (int t = 0; t < V; t++) {
             const int n = 8 * (cw + t);
             if (split) {
-                float4* dst = reinterpret_cast<float4*>(partials + ((int64_t)blockIdx.y * M + m) * N + n);
+                float4* dst = reinterpret_cast<float4*>(partials + ((int64_t)blockIdx.y * M_total + m) * N + n);
                 dst[0] = make_float4(y[t][0][r], y[t][1][r], y[t][2][r], y[t][3][r]);
                 dst[1] = make_float4(y[t][4][r], y[t][5][r], y[t][6][r], y[t][7][r]);
             } else {
@@ -558,7 +564,8 @@ DecodePlan make_decode_plan(int64_t N, int64_t K) {
     return p;
 }
 
-inline bool decode_path(int64_t M, int64_t group) { return M <= 16 && group == 128; }
+// The streaming kernel handles up to 64 tokens per weight pass as up to 4 slabs of 16.
+inline bool decode_path(int64_t M, int64_t group) { return M <= 64 && group == 128; }
 
 template <int V, int MT>
 void launch_awq(const AwqPlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
@@ -589,7 +596,7 @@ extern "C" size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
         const int64_t mm = M - m0 < 64 ? M - m0 : 64;
         const AwqPlan p = make_awq_plan(mm, N, K);  // sized for either kernel (the group size is not known here)
         size_t need = p.splits > 1 ? (size_t)p.splits * mm * N * sizeof(float) : 0;
-        if (mm <= 16 && K % 128 == 0) {
+        if (K % 128 == 0) {
             const DecodePlan d = make_decode_plan(N, K);
             const size_t need2 = d.splits > 1 ? (size_t)d.splits * mm * N * sizeof(float) : 0;
             if (need2 > need) need = need2;
@@ -628,10 +635,11 @@ extern "C" int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight,
             const DecodePlan d = make_decode_plan(N, K);
             splits = d.splits;
             if (splits > 1 && (!ws || workspace_bytes < (size_t)splits * mm * N * sizeof(float))) return LLMQ_ERR_WORKSPACE;
-            const dim3 grid(cdiv(Ni / 8, 16 * d.v), splits);
+            const int slabs = cdiv(mm, 16);
+            const dim3 grid(cdiv(Ni / 8, 16 * d.v) * slabs, splits);
 #define LLMQ_AWQ_DECODE(VV, KWW) \
     hipLaunchKernelGGL((awq_gemv_kernel<VV, KWW>), grid, dim3(KWW * kWave), 0, st, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, \
-                       Ki)
+                       Ki, slabs)
             if (d.v == 2) LLMQ_AWQ_DECODE(2, 4);
             else if (d.kw == 8) LLMQ_AWQ_DECODE(1, 8);
             else LLMQ_AWQ_DECODE(1, 4);
