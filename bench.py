@@ -48,6 +48,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-details", action="store_true", help="skip the per-shape FP8 / AWQ / layer tables")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--awq-only", action="store_true",
+                    help="profiler mode: only the W4A16 launches of configs[3] (4 projections x M in {1,4,16,64}), "
+                         "weights rotated beyond the Infinity Cache, preceded by one 256 MiB calibration copy")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant kernel's launches (for rocprofv3 summaries)")
     return ap.parse_args()
@@ -234,6 +237,39 @@ def details_awq(dev):
     return rows
 
 
+def awq_only(dev, steps, warmup):
+    """For profiler runs: the W4A16 launches of configs[3] in a fixed order, weights rotating through more than
+    256 MB per projection, after one plain copy of known size that calibrates the HBM byte counters."""
+    from llmqrt_amd import _abi, workloads as W
+    L = _abi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    cal_src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    launches, order = [], []
+    for pi, (pname, (K, N)) in enumerate(W.QWEN2_7B_PROJ.items()):
+        qw, qz, sc = W.awq_weights(N, K, W.seed_for(3, 100 + pi))
+        wbytes = qw.numel() * 4 + qz.numel() * 4 + sc.numel() * 2
+        ncopies = max(2, -(-320 * 1024 * 1024 // wbytes))
+        copies = [(qw.to(dev).clone(), qz.to(dev).clone(), sc.to(dev).clone()) for _ in range(ncopies)]
+        for mi, M in enumerate(W.AWQ_M):
+            x = W.activations(M, K, W.seed_for(3, 10 * pi + mi), dtype=torch.float16, outliers=False).to(dev)
+            out = torch.empty((M, N), dtype=torch.float16, device=dev)
+            wsp = torch.empty(max(L.llmq_awq_gemm_workspace_bytes(M, N, K), 16), dtype=torch.uint8, device=dev)
+            launches.append((x, out, wsp, copies, M, N, K))
+            order.append(f"{pname}_M{M}")
+    torch.cuda.synchronize()
+    for it in range(warmup + steps):
+        for (x, out, wsp, copies, M, N, K) in launches:
+            c = copies[it % len(copies)]
+            rc = L.llmq_awq_gemm(x.data_ptr(), K, c[0].data_ptr(), c[2].data_ptr(), c[1].data_ptr(), None, out.data_ptr(),
+                                 M, N, K, 128, wsp.data_ptr(), wsp.numel(), stream)
+            assert rc == 0
+    torch.cuda.synchronize()
+    print(json.dumps({"awq_only": True, "order": order, "steps": steps, "warmup": warmup,
+                      "calibration_copy_bytes_each_way": cal_src.numel() * 4}))
+
+
 def details_layer(dev):
     """Config 4: one decoder layer's linears (qkv, o, gate_up, down) in W8A8 with SmoothQuant factors
     (alpha = 0.5) folded into the preceding norm weight / the weights; prefill 2048 tokens and decode 32."""
@@ -324,6 +360,10 @@ def main():
     _abi.lib()
     stream_obj = torch.cuda.current_stream()
     stream = stream_obj.cuda_stream
+
+    if args.awq_only:
+        awq_only(dev, args.steps, args.warmup)
+        return
 
     linears = build_w8a8_sweep(dev)
     total_ops = sum(l.ops for l in linears)
