@@ -8,6 +8,7 @@ Layout:
   sq_fp8_kernels   drop-in for runtime.sq_fp8_kernels
   awq_kernels      drop-in for runtime.triton_kernels.awq_kernels
   linear/          quantized Linear modules + registry
+  fused_utils.py   fuse q/k/v or gate/up sibling modules into one
   workloads.py     seeded synthetic inputs of the benchmark configurations
 """
 __version__ = "0.1.0"
