@@ -9,6 +9,7 @@ Layout:
   awq_kernels      drop-in for runtime.triton_kernels.awq_kernels
   linear/          quantized Linear modules + registry
   fused_utils.py   fuse q/k/v or gate/up sibling modules into one
+  checkpoint.py    QuantConfig, nn.Linear replacement and by-name loading of safetensors checkpoints
   workloads.py     seeded synthetic inputs of the benchmark configurations
 """
 __version__ = "0.1.0"
