@@ -560,7 +560,11 @@ Plan make_plan(int64_t M, int64_t N, int64_t K) {
     double best_t = 1e300;
     for (const Model& md : kModels) {
         const TileShape s = kShapes[md.cfg];
-        if (M > 128 && md.cfg >= 4) continue;                 // skinny tiles are for decode-sized M
+        // skinny tiles are for small M; the 64-row tile also serves up to 1024 rows when 128x128 tiles
+        // could not even fill the CUs once and K is short (measured: o and qkv at M = 512)
+        if (M > 128 && md.cfg == 5) continue;
+        if (M > 128 && md.cfg == 4 &&
+            (M > 1024 || K > 8192 || (int64_t)cdiv(M, 128) * cdiv(N, 128) >= 2 * kNumCu)) continue;
         if (md.cfg < 5 && M <= s.bm / 2) continue;            // mostly padding
         const int64_t tiles = (int64_t)cdiv(M, s.bm) * cdiv(N, s.bn);
         for (int sp = 1; sp <= 16; sp++) {
@@ -582,12 +586,20 @@ Plan make_plan(int64_t M, int64_t N, int64_t K) {
 template <class C>
 int launch_cfg(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, int M, int N, int K, const Plan& p,
                const Epilogue& ep, void* out, int64_t ldo, void* acc_dump, void* ws, hipStream_t st) {
-    if (C::LDS_BYTES > 65536u &&
-        (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<C, true>),
-                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES) != hipSuccess ||
-         hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<C, false>),
-                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES) != hipSuccess))
-        return LLMQ_ERR_LAUNCH;
+    if (C::LDS_BYTES > 65536u) {
+        // tiles of more than 64 KB need the limit raised, once per kernel and device
+        static bool raised[64] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LLMQ_ERR_LAUNCH;
+        if (!raised[dev]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<C, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES) != hipSuccess ||
+                hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<C, false>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES) != hipSuccess)
+                return LLMQ_ERR_LAUNCH;
+            raised[dev] = true;  // benign if two threads race here: both set the same value
+        }
+    }
     const int tiles = cdiv(M, C::BM) * cdiv(N, C::BN);
     // every split covers whole K tiles -> the loads need no K predicate
     const bool kfull = (K % C::BK == 0) && (p.k_per_split % C::BK == 0);
