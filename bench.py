@@ -303,7 +303,25 @@ def details_layer(dev):
         per = {}
         for l in lins:
             per[l.name] = round(batch_time_us([lambda l=l: l.launch(stream)], stream_obj, 10), 2)
-        out.append({"M": M, "layer_linear_us": round(t, 2), "TOPS": round(ops / t / 1e6, 1), "per_linear_us": per})
+        row = {"M": M, "layer_linear_us": round(t, 2), "TOPS": round(ops / t / 1e6, 1), "per_linear_us": per}
+        if M <= 64:
+            # decode is launch-bound: the same eight kernels captured once into a HIP graph and replayed
+            # (the C ABI launches on the capturing stream and allocates nothing, so capture just works)
+            side = torch.cuda.Stream()
+            side.wait_stream(stream_obj)
+            with torch.cuda.stream(side):
+                s_side = side.cuda_stream
+                for l in lins:
+                    l.launch(s_side)
+                side.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    for l in lins:
+                        l.launch(torch.cuda.current_stream().cuda_stream)
+            stream_obj.wait_stream(side)
+            tg = batch_time_us([graph.replay], stream_obj, 10)
+            row["layer_linear_us_hip_graph"] = round(tg, 2)
+        out.append(row)
     return out
 
 

@@ -278,3 +278,47 @@ def test_fast_epilogue_is_bit_identical_to_the_general_one(cuda, force_plan, out
             fast8 = cutlass_f8f8bf16_tensorwise_sm89(*a8)
             general8 = cutlass_f8f8bf16_tensorwise_sm89(*a8, _acc_dump=dump8)
         assert torch.equal(fast8.view(torch.int16), general8.view(torch.int16)), f"fp8 cfg {cfg}"
+
+
+def test_hip_graph_replays_match_eager(cuda):
+    """The C ABI allocates nothing and launches on the stream it is given, so a decode-sized linear (quantizer +
+    split-K GEMM + its reduction kernel) can be captured into a HIP graph.  Every replay, with fresh inputs
+    and eager work of the same ops in between, must reproduce the eager result bit for bit."""
+    from llmqrt_amd import _abi, workloads as W
+    L = _abi.lib()
+    M, K, N = 16, 3584, 4608
+    qw, ws = W.int8_weights(N, K, 501)
+    qw, ws = qw.to(cuda), ws.to(cuda)
+    x = W.activations(M, K, 500).to(cuda)
+    qx = torch.empty((M, K), dtype=torch.int8, device=cuda)
+    sa = torch.empty(M, dtype=torch.float32, device=cuda)
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=cuda)
+    nws = L.llmq_gemm_workspace_bytes(M, N, K)
+    assert nws > 0, "the shape is meant to exercise the split-K path"
+    wsp = torch.empty(nws, dtype=torch.uint8, device=cuda)
+
+    def run(stream):
+        rc = L.llmq_quant_i8_per_token(x.data_ptr(), 0, M, K, K, qx.data_ptr(), sa.data_ptr(), 2, stream)
+        rc |= L.llmq_gemm_w8a8(qx.data_ptr(), K, qw.data_ptr(), K, sa.data_ptr(), ws.data_ptr(), 1.0, None, None, 0,
+                               0.0, out.data_ptr(), 0, N, M, N, K, None, wsp.data_ptr(), nws, stream)
+        assert rc == 0
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        run(side.cuda_stream)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            run(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    main = torch.cuda.current_stream().cuda_stream
+    for rep in range(4):
+        x.copy_(W.activations(M, K, 510 + rep).to(cuda))
+        run(main)
+        torch.cuda.synchronize()
+        eager = out.clone()
+        out.zero_()
+        wsp.fill_(0xFF)          # the workspace contents must not matter
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep}"
