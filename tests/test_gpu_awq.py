@@ -86,3 +86,25 @@ def test_gemm_asserts_like_reference(cuda):
         awq_gemm_triton(x[:, :64], qw, s, qz, split_k_iters=8)
     out = awq_gemm_triton(x, qw, s, qz, split_k_iters=8)    # all-zero q and z -> zeros
     assert torch.count_nonzero(out).item() == 0
+
+
+def test_gemm_random_shapes(cuda):
+    """Seeded random sizes: any M up to 70, N a multiple of 8, K a multiple of the group, groups 32 / 64 / 128."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    g = torch.Generator().manual_seed(777)
+    for case in range(24):
+        G = (32, 64, 128)[case % 3]
+        M = int(torch.randint(1, 71, (1,), generator=g))
+        N = 8 * int(torch.randint(1, 200, (1,), generator=g))
+        K = G * int(torch.randint(1, 1 + 2048 // G, (1,), generator=g))
+        qw, qz, sc = W.awq_weights(N, K, 9000 + case, group=G)
+        x = W.activations(M, K, 9100 + case, dtype=torch.float16, outliers=False)
+        bias = torch.randn(N, generator=g).half() if case % 2 else None
+        y = awq_gemm_triton(x.to(cuda), qw.to(cuda), sc.to(cuda), qz.to(cuda), split_k_iters=8,
+                            bias=None if bias is None else bias.to(cuda))
+        ref = R.awq_gemm(x, qw, qz, sc, G)
+        if bias is not None:
+            ref = (ref.float() + bias.float()).half()
+        rel = ((y.float().cpu() - ref.float()).abs().max() / ref.float().abs().max().clamp(min=1e-30)).item()
+        assert rel <= 1e-2, (case, M, N, K, G, rel)

@@ -322,3 +322,32 @@ def test_hip_graph_replays_match_eager(cuda):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager), f"replay {rep}"
+
+
+def test_w8a8_random_shapes(cuda):
+    """Seeded random problem sizes through the automatic plan: ragged M / N, every K that is a multiple of 16,
+    with and without bias, both output dtypes; int32 accumulators bit-exact, outputs within tolerance."""
+    from llmqrt_amd.sq_fp8_kernels import w8a8_int8_linear_bbf16_obf16_per_channel
+    g = torch.Generator().manual_seed(20240607)
+    for case in range(40):
+        M = int(torch.randint(1, 700, (1,), generator=g))
+        N = int(torch.randint(1, 900, (1,), generator=g))
+        K = 16 * int(torch.randint(1, 260, (1,), generator=g))
+        if case % 5 == 0:
+            M, N = M % 17 + 1, 8 * N      # decode-like
+        qx = torch.randint(-128, 128, (M, K), dtype=torch.int8, generator=g)
+        qw = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=g)
+        sx = torch.rand(M, generator=g) * 0.05 + 0.01
+        sw = torch.rand(N, generator=g) * 0.01 + 0.001
+        dtype = torch.bfloat16 if case % 2 else torch.float16
+        bias = torch.randn(N, generator=g).to(dtype)
+        acc_ref = R.int8_gemm_exact(qx, qw)
+        y_ref = R.w8a8_epilogue_per_token_per_channel(acc_ref, sx, sw, bias, dtype)
+        dump = torch.empty((M, N), dtype=torch.int32, device=cuda)
+        y = w8a8_int8_linear_bbf16_obf16_per_channel(qx.to(cuda), qw.to(cuda).t(), bias.to(cuda), sx.to(cuda).view(-1, 1),
+                                                     sw.to(cuda).view(1, -1), _acc_dump=dump)
+        assert torch.equal(dump.cpu(), acc_ref), (case, M, N, K)
+        assert rel_err(y, y_ref) <= REL_TOL, (case, M, N, K)
+        y2 = w8a8_int8_linear_bbf16_obf16_per_channel(qx.to(cuda), qw.to(cuda).t(), bias.to(cuda),
+                                                      sx.to(cuda).view(-1, 1), sw.to(cuda).view(1, -1))
+        assert torch.equal(y2.view(torch.int16), y.view(torch.int16)), (case, M, N, K)
