@@ -329,7 +329,8 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     // ---- epilogue.  The weights feed the MFMA row operand, so D is the transposed tile: a lane holds
     // token m = l32 and, in register r, channel 8*(r/4) + 4*khalf + r%4 -> 4 consecutive channels per
     // register quad.  After the dequant math the two half-waves exchange quads (v_permlane32_swap) so
-    // that every lane owns 8 consecutive channels of its token and stores them as one 16-byte vector.
+    // that every lane owns 8 consecutive channels of its token and stores them as one 16-byte vector,
+    // the two lanes of a token adjacent to each other.
     const bool split = gridDim.y > 1;
     const float alpha = ep.alpha * (ep.alpha_dev ? *ep.alpha_dev : 1.0f);
     const bool out_vec = ((ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(out) & 15u) == 0);
@@ -379,12 +380,12 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
                     for (int g = 0; g < 2; g++) {
 #pragma unroll
                         for (int x = 0; x < 2; x++) {
-                            const auto sw2 = __builtin_amdgcn_permlane32_swap(pk[g][x], pk[g + 2][x], false, false);
-                            pk[g][x] = sw2[0];
-                            pk[g + 2][x] = sw2[1];
+                            const auto sw2 = __builtin_amdgcn_permlane32_swap(pk[2 * g][x], pk[2 * g + 1][x], false, false);
+                            pk[2 * g][x] = sw2[0];
+                            pk[2 * g + 1][x] = sw2[1];
                         }
-                        *reinterpret_cast<uint4*>(orow + nb + 16 * khalf + 8 * g) =
-                            make_uint4(pk[g][0], pk[g][1], pk[g + 2][0], pk[g + 2][1]);
+                        *reinterpret_cast<uint4*>(orow + nb + 16 * g + 8 * khalf) =
+                            make_uint4(pk[2 * g][0], pk[2 * g][1], pk[2 * g + 1][0], pk[2 * g + 1][1]);
                     }
                 }
             }
@@ -449,19 +450,20 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
             }
             uint16_t* orow = reinterpret_cast<uint16_t*>(out) + (int64_t)m * ldo;
             if (full && out_vec) {
-                // lower half-wave keeps quads 0,1 and receives the upper half's quads 0,1 (channels +4..+7);
-                // upper half-wave keeps quads 2,3 and receives the lower half's quads 2,3
+                // quads 2g and 2g+1 are exchanged between the half-waves: the lower half ends up with
+                // channels 16g .. 16g+7 of its token, the upper half with 16g+8 .. 16g+15, so one store
+                // instruction writes 32 contiguous bytes per token row
 #pragma unroll
                 for (int g = 0; g < 2; g++) {
 #pragma unroll
                     for (int x = 0; x < 2; x++) {
-                        const auto sw2 = __builtin_amdgcn_permlane32_swap(pk[g][x], pk[g + 2][x], false, false);
-                        pk[g][x] = sw2[0];
-                        pk[g + 2][x] = sw2[1];
+                        const auto sw2 = __builtin_amdgcn_permlane32_swap(pk[2 * g][x], pk[2 * g + 1][x], false, false);
+                        pk[2 * g][x] = sw2[0];
+                        pk[2 * g + 1][x] = sw2[1];
                     }
                     if (m_ok)
-                        *reinterpret_cast<uint4*>(orow + nb + 16 * khalf + 8 * g) =
-                            make_uint4(pk[g][0], pk[g][1], pk[g + 2][0], pk[g + 2][1]);
+                        *reinterpret_cast<uint4*>(orow + nb + 16 * g + 8 * khalf) =
+                            make_uint4(pk[2 * g][0], pk[2 * g][1], pk[2 * g + 1][0], pk[2 * g + 1][1]);
                 }
             } else if (m_ok) {
 #pragma unroll
