@@ -51,6 +51,9 @@ def parse_args():
     ap.add_argument("--awq-only", action="store_true",
                     help="profiler mode: only the W4A16 launches of configs[3] (4 projections x M in {1,4,16,64}), "
                          "weights rotated beyond the Infinity Cache, preceded by one 256 MiB calibration copy")
+    ap.add_argument("--quant-only", action="store_true",
+                    help="profiler mode: only the row kernels (int8 / fp8 per-token quantizers, RMSNorm, RMSNorm fused "
+                         "with the int8 quantizer) at M in {2048, 8192} x K in {3584, 18944}, after one 256 MiB copy")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant kernel's launches (for rocprofv3 summaries)")
     return ap.parse_args()
@@ -270,6 +273,38 @@ def awq_only(dev, steps, warmup):
                       "calibration_copy_bytes_each_way": cal_src.numel() * 4}))
 
 
+def quant_only(dev, steps, warmup):
+    """For profiler runs: the HBM-bound row kernels in a fixed order after one calibration copy."""
+    from llmqrt_amd import _abi, workloads as W
+    L = _abi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    cal_src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    cases, order = [], []
+    for M in (2048, 8192):
+        for K in (3584, 18944):
+            x = W.activations(M, K, W.seed_for(1, 700 + M % 13 + K % 7)).to(dev)
+            w = torch.ones(K, dtype=torch.bfloat16, device=dev)
+            q = torch.empty((M, K), dtype=torch.int8, device=dev)
+            y = torch.empty_like(x)
+            sc = torch.empty(M, dtype=torch.float32, device=dev)
+            cases.append((x, w, q, y, sc, M, K))
+            order += [f"{k}_M{M}_K{K}" for k in ("quant_i8", "quant_fp8", "rmsnorm", "rmsnorm_quant_i8")]
+    torch.cuda.synchronize()
+    for _ in range(warmup + steps):
+        for (x, w, q, y, sc, M, K) in cases:
+            rc = L.llmq_quant_i8_per_token(x.data_ptr(), 0, M, K, K, q.data_ptr(), sc.data_ptr(), 2, stream)
+            rc |= L.llmq_quant_fp8_per_token(x.data_ptr(), 0, M, K, K, q.data_ptr(), sc.data_ptr(), stream)
+            rc |= L.llmq_rmsnorm(x.data_ptr(), 0, M, K, K, w.data_ptr(), 1e-6, y.data_ptr(), None, stream)
+            rc |= L.llmq_rmsnorm_quant_i8_per_token(x.data_ptr(), 0, M, K, K, w.data_ptr(), 1e-6, None, q.data_ptr(),
+                                                    sc.data_ptr(), 2, None, stream)
+            assert rc == 0
+    torch.cuda.synchronize()
+    print(json.dumps({"quant_only": True, "order": order, "steps": steps, "warmup": warmup,
+                      "calibration_copy_bytes_each_way": cal_src.numel() * 4}))
+
+
 def details_layer(dev):
     """Config 4: one decoder layer's linears (qkv, o, gate_up, down) in W8A8 with SmoothQuant factors
     (alpha = 0.5) folded into the preceding norm weight / the weights; prefill 2048 tokens and decode 32."""
@@ -381,6 +416,9 @@ def main():
 
     if args.awq_only:
         awq_only(dev, args.steps, args.warmup)
+        return
+    if args.quant_only:
+        quant_only(dev, args.steps, args.warmup)
         return
 
     linears = build_w8a8_sweep(dev)
