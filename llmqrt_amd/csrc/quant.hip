@@ -69,22 +69,24 @@ __device__ __forceinline__ uint2 quant8(uint4 raw, float s, float inv_s) {
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         float q = quotient<DT, QUOT>(f[i], s, inv_s);
-        const float c = __builtin_amdgcn_fmed3f(q, QP<MODE>::lo, QP<MODE>::hi);
-        f[i] = (q != q) ? q : c;  // clamp keeps NaN, as torch.clamp does
+        if (MODE == MODE_I8) {
+            f[i] = (q != q) ? 0.f : q;  // NaN narrows to 0 (what the reference's cast gives); clamp: see below
+        } else {
+            const float c = __builtin_amdgcn_fmed3f(q, QP<MODE>::lo, QP<MODE>::hi);
+            f[i] = (q != q) ? q : c;  // clamp keeps NaN, as torch.clamp does
+        }
     }
     uint32_t out[2];
     if (MODE == MODE_I8) {
 #pragma unroll
         for (int h = 0; h < 2; h++) {
-            uint32_t b[4];
+            // v_cvt_pk_u8_f32 rounds to the nearest integer (ties to even), saturates to [0, 255] and
+            // inserts the byte: with the value biased by 128 that is round + clamp(-128, 127) + pack in
+            // one instruction per element; the bias is taken out again by flipping the top bit of each byte
+            uint32_t w = 0;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                // adding 1.5*2^23 rounds to the nearest integer, ties to even, and leaves the
-                // two's-complement value in the low mantissa bits
-                const float v = f[4 * h + i];
-                b[i] = (v != v) ? 0u : (__float_as_uint(v + 12582912.0f) & 0xffu);
-            }
-            out[h] = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+            for (int i = 0; i < 4; i++) w = __builtin_amdgcn_cvt_pk_u8_f32(f[4 * h + i] + 128.0f, i, w);
+            out[h] = w ^ 0x80808080u;
         }
     } else {
 #pragma unroll
