@@ -109,19 +109,25 @@ def event_time_us(fn, stream_obj, reps):
 
 
 def batch_time_us(fns, stream_obj, reps, rounds=5):
-    """Median over `rounds` of the per-launch time of back-to-back launches cycling through `fns`."""
-    for f in fns:
-        f()
+    """Median over `rounds` batches of the per-launch time of back-to-back launches cycling through `fns`,
+    after 10 warm-up launches; short kernels (< 100 us) are timed over at least 100 launches per batch."""
+    for i in range(10):
+        fns[i % len(fns)]()
     stream_obj.synchronize()
     per = []
-    for _ in range(rounds):
+    for r in range(rounds + 1):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream_obj)
         for i in range(reps):
             fns[i % len(fns)]()
         e1.record(stream_obj)
         e1.synchronize()
-        per.append(e0.elapsed_time(e1) * 1e3 / reps)
+        t = e0.elapsed_time(e1) * 1e3 / reps
+        if r == 0:
+            if t < 100.0:
+                reps = max(reps, 100)
+            continue  # the first batch only sizes the later ones
+        per.append(t)
     return statistics.median(per)
 
 
