@@ -156,3 +156,13 @@ def test_rmsnorm_argument_validation_needs_no_gpu():
     assert L.llmq_rmsnorm_quant_i8_per_token(ok_ptr, 0, 4, 64, 64, ok_ptr, 1e-6, None, None, ok_ptr, 0, None, None) == -1
     assert L.llmq_rmsnorm_quant_i8_per_token(ok_ptr, 0, 4, 64, 64, ok_ptr, 1e-6, None, ok_ptr, ok_ptr, 1, None, None) == -2
     assert L.llmq_rmsnorm_quant_fp8_per_token(ok_ptr, 1, 4, 64, 32, ok_ptr, 1e-6, None, ok_ptr, ok_ptr, None, None) == -3
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more exits with a message instead of running."""
+    import subprocess
+    import sys
+    root = pathlib.Path(__file__).resolve().parent.parent
+    r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
