@@ -351,3 +351,30 @@ def test_w8a8_random_shapes(cuda):
         y2 = w8a8_int8_linear_bbf16_obf16_per_channel(qx.to(cuda), qw.to(cuda).t(), bias.to(cuda),
                                                       sx.to(cuda).view(-1, 1), sw.to(cuda).view(1, -1))
         assert torch.equal(y2.view(torch.int16), y.view(torch.int16)), (case, M, N, K)
+
+
+def test_w8a8_full_prefill_size_properties(cuda):
+    """The largest launch of the benchmark (M = 8192, N = 37888, K = 3584): 48 sampled token rows of the int32
+    accumulators against the exact integer GEMM, the fast epilogue equal to the general one on every element,
+    and a size-independent property on all 310 M outputs: doubling the activation scales doubles the result."""
+    from llmqrt_amd.sq_fp8_kernels import w8a8_int8_linear_bbf16_obf16_per_channel
+    M, N, K = 8192, 37888, 3584
+    g = torch.Generator().manual_seed(99)
+    qx = torch.randint(-128, 128, (M, K), dtype=torch.int8, generator=g)
+    qw = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=g)
+    sx = torch.rand(M, generator=g) * 0.05 + 0.01
+    sw = torch.rand(N, generator=g) * 0.01 + 0.001
+    bias0 = torch.zeros(N, dtype=torch.bfloat16, device=cuda)
+    a, b = qx.to(cuda), qw.to(cuda).t()
+    sxd, swd = sx.to(cuda).view(-1, 1), sw.to(cuda).view(1, -1)
+    dump = torch.empty((M, N), dtype=torch.int32, device=cuda)
+    general = w8a8_int8_linear_bbf16_obf16_per_channel(a, b, bias0, sxd, swd, _acc_dump=dump)
+    fast = w8a8_int8_linear_bbf16_obf16_per_channel(a, b, bias0, sxd, swd)
+    assert torch.equal(fast.view(torch.int16), general.view(torch.int16))
+    rows = torch.arange(5, M, M // 48)
+    acc_ref = R.int8_gemm_exact(qx[rows], qw)
+    assert torch.equal(dump[rows.to(cuda)].cpu(), acc_ref)
+    y_ref = R.w8a8_epilogue_per_token_per_channel(acc_ref, sx[rows], sw, None, torch.bfloat16)
+    assert rel_err(fast[rows.to(cuda)], y_ref) <= REL_TOL
+    doubled = w8a8_int8_linear_bbf16_obf16_per_channel(a, b, bias0, 2 * sxd, swd)
+    assert torch.equal(doubled, 2 * fast)

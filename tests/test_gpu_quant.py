@@ -130,3 +130,23 @@ def test_empty_rows(cuda):
     assert q.shape == (0, 64) and s.shape == (0, 1)
     q, s = per_token_quantize(x)
     assert q.shape == (0, 64) and s.shape == (0, 1)
+
+
+def test_full_size_scaling_property(cuda):
+    """Largest quantizer launch of the benchmark (M = 8192, K = 18944), checked through a size-independent
+    property instead of the CPU oracle: multiplying the input by 2 is exact in bf16, leaves every code
+    unchanged and doubles every scale; a sample of rows is also compared with the oracle bit for bit."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.quantize import per_token_quantize, quantize_activation_per_token_absmax
+    M, K = 8192, 18944
+    x = W.activations(M, K, 4321).to(cuda)
+    for quant in (quantize_activation_per_token_absmax, per_token_quantize):
+        q1, s1 = quant(x)
+        q2, s2 = quant(x * 2)
+        assert torch.equal(q1.view(torch.uint8), q2.view(torch.uint8))
+        assert torch.equal(s2.float(), 2 * s1.float())
+    rows = torch.arange(3, M, M // 32)
+    xr = x[rows.to(cuda)].cpu()
+    q_ref, s_ref = R.quantize_activation_per_token_absmax(xr)
+    q, s = quantize_activation_per_token_absmax(x)
+    assert torch.equal(q[rows.to(cuda)].cpu(), q_ref) and torch.equal(s[rows.to(cuda)].cpu().view(torch.int16), s_ref.view(torch.int16))
