@@ -108,3 +108,23 @@ def test_gemm_random_shapes(cuda):
             ref = (ref.float() + bias.float()).half()
         rel = ((y.float().cpu() - ref.float()).abs().max() / ref.float().abs().max().clamp(min=1e-30)).item()
         assert rel <= 1e-2, (case, M, N, K, G, rel)
+
+
+@pytest.mark.parametrize("K", [512, 8320])
+def test_module_paths_agree_around_the_token_threshold(cuda, K):
+    """WQLinear_GEMM switches from the fused kernel to dequantize + matmul at a measured token count; one token
+    below and at the threshold both paths must meet the same bound against the oracle."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.linear import WQLinear_GEMM
+    from llmqrt_amd.linear.linear_awq import dequant_matmul_token_threshold
+    N = 264
+    qw, qz, sc = W.awq_weights(N, K, 4242)
+    m = WQLinear_GEMM(4, 128, K, N, False, cuda)
+    m.qweight, m.qzeros, m.scales = qw.to(cuda), qz.to(cuda), sc.to(cuda)
+    t = dequant_matmul_token_threshold(K)
+    assert t < 1024
+    for M in (t - 1, t):
+        x = W.activations(M, K, 4300 + M, dtype=torch.float16, outliers=False)
+        y = m(x.to(cuda).view(1, M, K))
+        assert y.shape == (1, M, N) and y.dtype == torch.float16
+        assert rel_err(y.view(M, N), R.awq_gemm(x, qw, qz, sc, 128)) <= REL_TOL
