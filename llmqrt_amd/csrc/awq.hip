@@ -520,6 +520,45 @@ __global__ __launch_bounds__(256) void awq_dequant_kernel(const uint32_t* __rest
     }
 }
 
+// Dequantizer for group sizes that are multiples of 8 (all real checkpoints): a wavefront owns 64 word
+// columns x 8 consecutive K rows, which lie in one group, so zeros and scales are loaded once per 8 words
+// and all 8 word loads are in flight together.  Nibbles p and p + 4 of a word are adjacent columns, so one
+// shift + mask yields two columns as the fp16 pair (1024 + q_lo, 1024 + q_hi); subtracting (1024 + z) is
+// exact and the packed fp16 multiply by the scale pair rounds once, like the scalar kernel above.
+__global__ __launch_bounds__(256) void awq_dequant_rows_kernel(const uint32_t* __restrict__ qw,
+                                                               const uint16_t* __restrict__ scales,
+                                                               const uint32_t* __restrict__ qz,
+                                                               uint16_t* __restrict__ out, int K, int Nw, int G) {
+    constexpr int R = 8;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int c = blockIdx.x * kWave + lane;
+    const int k0 = ((int)blockIdx.y * 4 + wave) * R;
+    if (c >= Nw || k0 >= K) return;
+    const int64_t g = k0 / G;
+    uint32_t w[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) w[r] = qw[(int64_t)(k0 + r) * Nw + c];
+    const uint32_t z = qz[g * Nw + c];
+    const uint4 sv = *reinterpret_cast<const uint4*>(scales + (g * Nw + c) * 8);
+    const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w};
+    h2 zp[4], sp[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        zp[j] = __builtin_bit_cast(h2, ((z >> (4 * j)) & 0x000F000Fu) | 0x64006400u);
+        sp[j] = __builtin_bit_cast(h2, sw[j]);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const h2 q = __builtin_bit_cast(h2, ((w[r] >> (4 * j)) & 0x000F000Fu) | 0x64006400u);
+            o[j] = __builtin_bit_cast(uint32_t, (q - zp[j]) * sp[j]);
+        }
+        *reinterpret_cast<uint4*>(out + ((int64_t)(k0 + r) * Nw + c) * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
 struct AwqPlan { int v, mt, splits, chunks_per_block; };
 
 inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
@@ -672,6 +711,13 @@ extern "C" int llmq_awq_dequant(const int32_t* qweight, const void* scales, cons
     if ((N & 7) || group <= 0 || (K % group) || N > 0x7fffffffLL) return LLMQ_ERR_SHAPE;
     if (!aligned16(scales) || !aligned16(out)) return LLMQ_ERR_ALIGN;
     const int64_t total = K * (N / 8);
+    if (group % 8 == 0 && K <= 0x7fffffffLL && (K / 8 + 3) / 4 <= 65535) {
+        const dim3 grid((unsigned)((N / 8 + kWave - 1) / kWave), (unsigned)((K / 8 + 3) / 4));
+        hipLaunchKernelGGL(awq_dequant_rows_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const uint32_t*)qweight,
+                           (const uint16_t*)scales, (const uint32_t*)qzeros, (uint16_t*)out, (int)K, (int)(N / 8),
+                           (int)group);
+        return launch_status();
+    }
     const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
     hipLaunchKernelGGL(awq_dequant_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const uint32_t*)qweight,
                        (const uint16_t*)scales, (const uint32_t*)qzeros, (uint16_t*)out, K, (int)(N / 8), (int)group);

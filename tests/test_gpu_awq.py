@@ -18,7 +18,8 @@ def rel_err(y, ref):
     return ((y - ref).abs().max() / ref.abs().max().clamp(min=1e-30)).item()
 
 
-@pytest.mark.parametrize("K,N,G", [(3584, 4608, 128), (896, 4864, 128), (256, 264, 64), (128, 8, 32), (512, 1000, 512)])
+@pytest.mark.parametrize("K,N,G", [(3584, 4608, 128), (896, 4864, 128), (256, 264, 64), (128, 8, 32), (512, 1000, 512),
+                                   (8, 520, 8), (12, 1000, 12), (20, 8, 20)])  # the last two: one group that is not a multiple of 8
 def test_dequant_bit_exact(cuda, K, N, G):
     from llmqrt_amd import workloads as W
     from llmqrt_amd.awq_kernels import awq_dequantize_triton
