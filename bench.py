@@ -242,6 +242,24 @@ def details_awq(dev):
             rows.append({"proj": pname, "M": M, "us_hbm": round(t_rot, 2), "us_cache_resident": round(t_res, 2),
                          "GBs_hbm": round(b / t_rot / 1e3, 1), "pct_hbm_peak": round(100 * b / t_rot / 1e3 / PEAK_HBM_GBS, 2),
                          "GBs_cache_resident": round(b / t_res / 1e3, 1), "weight_copies_rotated": ncopies})
+        # prefill side of the module: the dequantizer (weights resident), alone and followed by the fp16 matmul
+        deq = torch.empty((K, N), dtype=torch.float16, device=dev)
+        c = copies[0]
+
+        def dequant():
+            L.llmq_awq_dequant(c[0].data_ptr(), c[2].data_ptr(), c[1].data_ptr(), deq.data_ptr(), K, N, 128, stream)
+        t_deq = batch_time_us([dequant], stream_obj, 40)
+        xp = W.activations(2048, K, W.seed_for(3, 900 + pi), dtype=torch.float16, outliers=False).to(dev)
+
+        def prefill():
+            dequant()
+            torch.matmul(xp, deq)
+        t_pre = batch_time_us([prefill], stream_obj, 10)
+        db = K * N // 2 + 2 * K * N
+        rows.append({"proj": pname, "dequant_us": round(t_deq, 2), "dequant_GBs": round(db / t_deq / 1e3, 1),
+                     "dequant_pct_hbm_peak": round(100 * db / t_deq / 1e3 / PEAK_HBM_GBS, 2),
+                     "prefill_M2048_dequant_plus_fp16_matmul_us": round(t_pre, 1),
+                     "prefill_M2048_TFLOPs": round(2 * 2048 * N * K / t_pre / 1e6, 1)})
         del copies
     return rows
 
