@@ -166,7 +166,7 @@ int llmq_gemm_num_configs(void);
 /* out[m,n] = fp16( sum_k x[m,k] * fp16((q[k,n] - z[k/G,n]) * s[k/G,n]) + bias[n] ), fp32
  * accumulation in a fixed order (deterministic, unlike the reference's fp16 atomics).
  * x: fp16 [M,K] (ldx >= K, K % 32 == 0); out: fp16 [M,N] contiguous; bias: fp16 [N] or NULL.
- * For M <= 16 and group 128 the weights enter the matrix core unrounded (exact (q - z) * s in
+ * For M <= 64 and group 128 the weights enter the matrix core unrounded (exact (q - z) * s in
  * fp32) instead of rounded to fp16 first; both are within 1e-2 of the dequantize-then-matmul math.
  * workspace: >= llmq_awq_gemm_workspace_bytes(M,N,K) bytes, 16-byte aligned, contents irrelevant. */
 int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight, const void* scales,

@@ -254,7 +254,7 @@ __global__ __launch_bounds__(kBlockWaves * kWave) void awq_gemm_kernel(
     }
 }
 
-// Decode kernel (M <= 16, group size 128).  Same streaming scheme, with the scale and the zero point
+// Decode kernel (16 tokens per block, up to 4 such slabs per launch; group size 128).  Same streaming scheme, with the scale and the zero point
 // moved out of the per-weight work.  The raw nibbles go to the matrix core as fp16 SUBNORMALS:
 // (u & 0x000F000F) read as two fp16 values is q * 2^-24 (a high nibble, u & 0x00F000F0, is
 // 16 q * 2^-24); their products with fp16 activations are exact in the fp32 accumulator.  Per
@@ -584,7 +584,7 @@ AwqPlan make_awq_plan(int64_t M, int64_t N, int64_t K) {
     return p;
 }
 
-// Decode kernel (M <= 16, group 128): a block = one column tile x KW wavefronts along K; a K split
+// Decode kernel (group 128): a block = one column tile x one 16-token slab x KW wavefronts along K; a K split
 // across blocks only when the tiles alone cannot fill the GPU.
 struct DecodePlan { int v, kw, splits; };
 DecodePlan make_decode_plan(int64_t N, int64_t K) {
