@@ -23,6 +23,14 @@
 #include "llmq_common.h"
 
 namespace llmq {
+
+// Tile kernel for many tokens (awq_tile.hip).
+struct AwqTilePlan { int cfg, splits, k_per_split; };
+AwqTilePlan make_awq_tile_plan(int64_t M, int64_t N, int64_t K, int force_cfg, int force_splits);
+int launch_awq_tile(const AwqTilePlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
+                    const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K, int G,
+                    hipStream_t st);
+
 namespace {
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
@@ -606,6 +614,13 @@ DecodePlan make_decode_plan(int64_t N, int64_t K) {
 // The streaming kernel handles up to 64 tokens per weight pass as up to 4 slabs of 16.
 inline bool decode_path(int64_t M, int64_t group) { return M <= 64 && group == 128; }
 
+// More than 64 tokens go to the tile kernel (weights dequantized once per token tile on their way into LDS);
+// llmq_awq_force_plan(3 | 4, ...) forces its 64x128 | 256x256 tile for any M, (1 | 2, ...) keeps the slabs.
+inline bool tile_path(int64_t M) { return g_force_v >= 3 || (g_force_v == 0 && M > 64); }
+inline AwqTilePlan tile_plan(int64_t M, int64_t N, int64_t K) {
+    return make_awq_tile_plan(M, N, K, g_force_v >= 3 ? g_force_v - 3 : -1, g_force_splits);
+}
+
 template <int V, int MT>
 void launch_awq(const AwqPlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
                 const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K, int G,
@@ -621,7 +636,7 @@ void launch_awq(const AwqPlan& p, const uint16_t* x, int64_t ldx, const uint32_t
 using namespace llmq;
 
 extern "C" int llmq_awq_force_plan(int v, int splits, int k_waves) {
-    if (v < 0 || v > 2 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
+    if (v < 0 || v > 4 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
     g_force_v = v;
     g_force_splits = splits;
     g_force_kw = k_waves;
@@ -631,6 +646,10 @@ extern "C" int llmq_awq_force_plan(int v, int splits, int k_waves) {
 extern "C" size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     size_t total = 0;
+    if (tile_path(M)) {
+        const AwqTilePlan t = tile_plan(M, N, K);
+        if (t.splits > 1) total = (size_t)t.splits * M * N * sizeof(float);
+    }
     for (int64_t m0 = 0; m0 < M; m0 += 64) {
         const int64_t mm = M - m0 < 64 ? M - m0 : 64;
         const AwqPlan p = make_awq_plan(mm, N, K);  // sized for either kernel (the group size is not known here)
@@ -664,6 +683,20 @@ extern "C" int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight,
     const uint16_t* sc = (const uint16_t*)scales;
     const uint16_t* bs = (const uint16_t*)bias;
     const int Ni = (int)N, Ki = (int)K, Gi = (int)group;
+    if (tile_path(M)) {
+        const AwqTilePlan t = tile_plan(M, N, K);
+        if (t.splits > 1 && (!ws || workspace_bytes < (size_t)t.splits * M * N * sizeof(float))) return LLMQ_ERR_WORKSPACE;
+        const int rc = launch_awq_tile(t, (const uint16_t*)x, ldx, qw, sc, qz, bs, (uint16_t*)out, ws, (int)M, Ni, Ki, Gi, st);
+        if (rc != LLMQ_OK) return rc;
+        if (t.splits > 1) {
+            const int64_t total = M * N;
+            const int blocks = (int)((total + 255) / 256 < 2048 ? (total + 255) / 256 : 2048);
+            hipLaunchKernelGGL(awq_finish_kernel, dim3(blocks), dim3(256), 0, st, ws, t.splits, total, Ni, bs,
+                               (uint16_t*)out);
+            if (launch_status() != LLMQ_OK) return LLMQ_ERR_LAUNCH;
+        }
+        return LLMQ_OK;
+    }
     // tokens are processed in slabs of at most 64 rows (4 MFMA token tiles per weight pass)
     for (int64_t m0 = 0; m0 < M; m0 += 64) {
         const int mm = (int)(M - m0 < 64 ? M - m0 : 64);

@@ -129,3 +129,51 @@ def test_module_paths_agree_around_the_token_threshold(cuda, K):
         y = m(x.to(cuda).view(1, M, K))
         assert y.shape == (1, M, N) and y.dtype == torch.float16
         assert rel_err(y.view(M, N), R.awq_gemm(x, qw, qz, sc, 128)) <= REL_TOL
+
+
+@pytest.fixture
+def force_awq_plan():
+    from llmqrt_amd import _abi
+    yield lambda v, splits: _abi.check(_abi.lib().llmq_awq_force_plan(v, splits, 0), "llmq_awq_force_plan")
+    _abi.lib().llmq_awq_force_plan(0, 0, 0)
+
+
+# (M, K, N, G): ragged token / channel edges, K with a half tile at the end (K % 64 == 32), one K tile,
+# groups of 32 (two per K tile) / 64 / 128 / K, more than one token tile and more than one channel tile
+TILE_SHAPES = [(300, 1056, 520, 32), (65, 64, 8, 64), (1, 96, 136, 32), (257, 512, 264, 512), (130, 3584, 4608, 128),
+               (64, 1024, 1000, 128)]
+
+
+@pytest.mark.parametrize("tile", [3, 4])
+@pytest.mark.parametrize("splits", [0, 1, 3])
+@pytest.mark.parametrize("M,K,N,G", TILE_SHAPES)
+def test_tile_kernel_every_shape_and_split(cuda, force_awq_plan, tile, splits, M, K, N, G):
+    """The many-token tile kernel (both tile shapes, fused and split-K) against the oracle.  Its weights are
+    fp16((q - z) * s) as in the reference dequantizer, accumulated in fp32."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    qw, qz, s = W.awq_weights(N, K, 7 * M + N, group=G)
+    x = W.activations(M, K, 8 * M + K, dtype=torch.float16, outliers=False)
+    bias = (0.1 * torch.randn(N, generator=torch.Generator().manual_seed(M))).half() if splits != 1 else None
+    ref = R.awq_gemm(x, qw, qz, s, G)
+    if bias is not None:
+        ref = (ref.float() + bias.float()).half()
+    force_awq_plan(tile, splits)
+    out = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8,
+                          bias=None if bias is None else bias.to(cuda))
+    assert out.shape == (M, N) and out.dtype == torch.float16
+    assert rel_err(out, ref) <= REL_TOL, (tile, splits, M, K, N, G)
+    out2 = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8,
+                           bias=None if bias is None else bias.to(cuda))
+    assert torch.equal(out, out2), "deterministic"
+
+
+def test_tile_kernel_prefill_size(cuda):
+    """1024 tokens of the Qwen2-7B qkv projection through the default plan (256x256 tiles)."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    M, K, N = 1024, 3584, 4608
+    qw, qz, s = W.awq_weights(N, K, 515)
+    x = W.activations(M, K, 516, dtype=torch.float16, outliers=False)
+    out = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8)
+    assert rel_err(out, R.awq_gemm(x, qw, qz, s, 128)) <= REL_TOL
