@@ -279,13 +279,19 @@ __global__ __launch_bounds__(kBlockWaves * kWave) void awq_gemm_kernel(
 // unconditionally (indices clamped to the wavefront's last group) so that the compiler can count the
 // loads in flight and wait only for the oldest ring slot; 4 chunks (+ the next group's zeros/scales)
 // stay in flight per wavefront.
-template <int V, int KW>
+template <int V, int KW, int MS>
 __global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, const uint32_t* __restrict__ qw,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qz, const uint16_t* __restrict__ bias,
     uint16_t* __restrict__ out, float* __restrict__ partials, int M_total, int N, int K, int slabs) {
     typedef typename WordVec<V>::type wvec;
-    constexpr int G = 128, RING = G / kChunkK, NACC = V * 8;
+    constexpr int G = 128, RING = G / kChunkK, NACC = MS * V * 8;
+    constexpr int TOK = 16 * MS;  // tokens per block: MS MFMA token tiles share every unpacked weight operand
+    // With several token tiles the per-group rescaling of the accumulators (two fused multiply-adds per
+    // accumulator element and group, plus the moves between the two register files) outweighs what the
+    // subnormal operands save in unpacking: those variants dequantize each weight to fp16((q - z) * s), as
+    // the reference dequantizer rounds it, and accumulate straight into y.
+    constexpr bool EX = MS > 1;
     __shared__ float4 red[(KW / 2) * NACC * kWave];
 
     const int lane = threadIdx.x & (kWave - 1);
@@ -302,10 +308,10 @@ __global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
         seq = xcd < r ? xcd * (q + 1) + local : r * (q + 1) + (xcd - r) * q + local;
     }
     const int tile = seq / slabs, slab = seq - tile * slabs;
-    const int M = min(16, M_total - 16 * slab);  // tokens of this slab
-    x += (int64_t)(16 * slab) * ldx;
-    out += (int64_t)(16 * slab) * N;
-    partials += (int64_t)(16 * slab) * N;
+    const int M = min(TOK, M_total - TOK * slab);  // tokens of this slab
+    x += (int64_t)(TOK * slab) * ldx;
+    out += (int64_t)(TOK * slab) * N;
+    partials += (int64_t)(TOK * slab) * N;
     const int cw = tile * (16 * V) + V * li;  // first word column of this lane
     const bool col_ok = cw < Nw;
     const int cwc = col_ok ? cw : 0;
@@ -317,29 +323,37 @@ __global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
     const int gstride = (int)gridDim.y * KW;
     const int g0 = (int)blockIdx.y * KW + wave;
 
-    v4f y[V][8], accg[V][8], xs = v4f{0.f, 0.f, 0.f, 0.f};
+    v4f y[MS][V][8], accg[MS][V][8], xs[MS];
 #pragma unroll
-    for (int t = 0; t < V; t++)
+    for (int a = 0; a < MS; a++) {
+        xs[a] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            y[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
-            accg[t][j] = v4f{0.f, 0.f, 0.f, 0.f};
-        }
+        for (int t = 0; t < V; t++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                y[a][t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+                accg[a][t][j] = v4f{0.f, 0.f, 0.f, 0.f};
+            }
+    }
 
     if (g0 < ngroups) {
         wvec wr[RING][8];
-        uint4 xr[RING];
+        uint4 xr[RING][MS];
         uint32_t voff[8];  // loop-invariant row offsets; the chunk base is wave-uniform
 #pragma unroll
         for (int r = 0; r < 8; r++) voff[r] = (uint32_t)(((8 * kb + r) * Nw + cwc) * 4);
-        const uint32_t xoff = (uint32_t)((min(li, M - 1) * (int)ldx + 8 * kb) * 2);
+        uint32_t xoff[MS];
+#pragma unroll
+        for (int a = 0; a < MS; a++) xoff[a] = (uint32_t)((min(16 * a + li, M - 1) * (int)ldx + 8 * kb) * 2);
         // loads past the last group of this wavefront re-read that group (results unused): no branches
-        auto load_chunk = [&](int g, int u, wvec* wdst, uint4& xdst) {
+        auto load_chunk = [&](int g, int u, wvec* wdst, uint4* xdst) {
             const int c = (g < ngroups ? g : g - gstride) * RING + u;
             const uint8_t* wbase = reinterpret_cast<const uint8_t*>(qw) + (int64_t)c * kChunkK * Nw * 4;
 #pragma unroll
             for (int r = 0; r < 8; r++) wdst[r] = *reinterpret_cast<const wvec*>(wbase + voff[r]);
-            xdst = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(x) + (int64_t)c * kChunkK * 2 + xoff);
+#pragma unroll
+            for (int a = 0; a < MS; a++)
+                xdst[a] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(x) + (int64_t)c * kChunkK * 2 + xoff[a]);
         };
         wvec z_cur, z_next;
         uint4 s_cur[V], s_next[V];
@@ -352,7 +366,11 @@ __global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
         };
         const h8 ones = {(_Float16)1.f, (_Float16)1.f, (_Float16)1.f, (_Float16)1.f,
                          (_Float16)1.f, (_Float16)1.f, (_Float16)1.f, (_Float16)1.f};
-        const bool row_ok = li < M;
+        uint32_t magic = 0x64006400u;
+        asm volatile("" : "+v"(magic));  // opaque: (u & mask) | magic stays one v_and_or_b32
+        bool row_ok[MS];
+#pragma unroll
+        for (int a = 0; a < MS; a++) row_ok[a] = 16 * a + li < M;
 
         // same issue order as in the loop (group, slot 0..3), pinned, so that the wait counts the compiler
         // derives at the loop head are those of the steady state
@@ -370,32 +388,69 @@ __global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
 #pragma unroll
             for (int t = 0; t < V; t++) s_cur[t] = s_next[t];
             load_group(g + gstride);
+            h2 cz[V][8], s2[V][8];  // EX: -(1024 + z) or -(64 + z), and the scale, both halves equal
+            if constexpr (EX) {
+#pragma unroll
+                for (int t = 0; t < V; t++) {
+                    const uint32_t zw = word_of<V>(z_cur, t);
+                    const uint32_t sw[4] = {s_cur[t].x, s_cur[t].y, s_cur[t].z, s_cur[t].w};
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const int p = rev_nibble(j);
+                        const uint32_t z = (zw >> (4 * p)) & 0xFu;
+                        const uint32_t c16 = (p & 1) ? (0xD400u | (z << 4)) : (0xE400u | z);
+                        cz[t][j] = __builtin_bit_cast(h2, c16 * 0x00010001u);
+                        const uint32_t sh = (j & 1) ? (sw[j >> 1] >> 16) : (sw[j >> 1] & 0xffffu);
+                        s2[t][j] = __builtin_bit_cast(h2, sh * 0x00010001u);
+                    }
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int u = 0; u < RING; u++) {
-                uint4 xv = xr[u];
-                if (!row_ok) xv = make_uint4(0, 0, 0, 0);
-                const h8 xb = __builtin_bit_cast(h8, xv);
-                xs = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb, ones, xs, 0, 0, 0);
+                h8 xb[MS];
+#pragma unroll
+                for (int a = 0; a < MS; a++) {
+                    uint4 xv = xr[u][a];
+                    if (!row_ok[a]) xv = make_uint4(0, 0, 0, 0);
+                    xb[a] = __builtin_bit_cast(h8, xv);
+                    if constexpr (!EX) xs[a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[a], ones, xs[a], 0, 0, 0);
+                }
 #pragma unroll
                 for (int t = 0; t < V; t++) {
 #pragma unroll
                     for (int bsel = 0; bsel < 4; bsel++) {  // byte of the word: nibbles 2*bsel (low), 2*bsel+1 (high)
                         const uint32_t sel = (uint32_t)bsel | 0x0c00u | ((uint32_t)(4 + bsel) << 16) | 0x0c000000u;
+                        constexpr int kColOfNibble[8] = {0, 2, 4, 6, 1, 3, 5, 7};  // logical column of nibble p
+                        const int jl = kColOfNibble[2 * bsel], jh = kColOfNibble[2 * bsel + 1];
                         uint32_t lo[4], hi[4];
 #pragma unroll
                         for (int pr = 0; pr < 4; pr++) {
                             const uint32_t w0 = word_of<V>(wr[u][2 * pr], t), w1 = word_of<V>(wr[u][2 * pr + 1], t);
                             const uint32_t uu = __builtin_amdgcn_perm(w1, w0, sel);  // byte0 <- w0, byte2 <- w1
-                            lo[pr] = uu & 0x000F000Fu;                               // q * 2^-24 as fp16 subnormals
-                            hi[pr] = uu & 0x00F000F0u;                               // 16 q * 2^-24
+                            if constexpr (EX) {
+                                const h2 hl = __builtin_bit_cast(h2, (uu & 0x000F000Fu) | magic);  // 1024 + q
+                                const h2 hh = __builtin_bit_cast(h2, (uu & 0x00F000F0u) | magic);  // 1024 + 16 q
+                                const h2 k16 = {(_Float16)0.0625f, (_Float16)0.0625f};
+                                lo[pr] = __builtin_bit_cast(uint32_t, (hl + cz[t][jl]) * s2[t][jl]);
+                                hi[pr] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(hh, k16, cz[t][jh]) * s2[t][jh]);
+                            } else {
+                                lo[pr] = uu & 0x000F000Fu;  // q * 2^-24 as fp16 subnormals
+                                hi[pr] = uu & 0x00F000F0u;  // 16 q * 2^-24
+                            }
                         }
-                        constexpr int kColOfNibble[8] = {0, 2, 4, 6, 1, 3, 5, 7};  // logical column of nibble p
-                        const int jl = kColOfNibble[2 * bsel], jh = kColOfNibble[2 * bsel + 1];
                         const h8 bl = __builtin_bit_cast(h8, v4i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3]});
                         const h8 bh = __builtin_bit_cast(h8, v4i{(int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]});
-                        accg[t][jl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb, bl, accg[t][jl], 0, 0, 0);
-                        accg[t][jh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb, bh, accg[t][jh], 0, 0, 0);
+#pragma unroll
+                        for (int a = 0; a < MS; a++) {
+                            if constexpr (EX) {
+                                y[a][t][jl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[a], bl, y[a][t][jl], 0, 0, 0);
+                                y[a][t][jh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[a], bh, y[a][t][jh], 0, 0, 0);
+                            } else {
+                                accg[a][t][jl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[a], bl, accg[a][t][jl], 0, 0, 0);
+                                accg[a][t][jh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[a], bh, accg[a][t][jh], 0, 0, 0);
+                            }
+                        }
                     }
                 }
                 // keep the issue order: this slot's refill goes out only now, and nothing of the next
@@ -405,6 +460,7 @@ __global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
                 __builtin_amdgcn_sched_barrier(0);
             }
             // y += s * 2^24 * acc - s * z * xsum for this group; the group accumulators restart at 0
+            if constexpr (!EX) {
 #pragma unroll
             for (int t = 0; t < V; t++) {
                 const uint32_t zw = word_of<V>(z_cur, t);
@@ -417,13 +473,17 @@ __global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
                     const float s1 = sf * ((p & 1) ? 1048576.0f : 16777216.0f);  // 2^20 for 16 q, 2^24 for q
                     const float sz = -sf * zf;
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        y[t][j][r] = fmaf(s1, accg[t][j][r], fmaf(sz, xs[r], y[t][j][r]));
-                        accg[t][j][r] = 0.f;
-                    }
+                    for (int a = 0; a < MS; a++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            y[a][t][j][r] = fmaf(s1, accg[a][t][j][r], fmaf(sz, xs[a][r], y[a][t][j][r]));
+                            accg[a][t][j][r] = 0.f;
+                        }
                 }
             }
-            xs = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int a = 0; a < MS; a++) xs[a] = v4f{0.f, 0.f, 0.f, 0.f};
+            }
         }
     }
 
@@ -433,51 +493,58 @@ __global__ __launch_bounds__(KW * kWave) void awq_gemv_kernel(
         __syncthreads();
         if (wave >= half && wave < 2 * half) {
 #pragma unroll
-            for (int t = 0; t < V; t++)
+            for (int a = 0; a < MS; a++)
 #pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const v4f v = y[t][j];
-                    red[((wave - half) * NACC + t * 8 + j) * kWave + lane] = make_float4(v[0], v[1], v[2], v[3]);
-                }
+                for (int t = 0; t < V; t++)
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const v4f v = y[a][t][j];
+                        red[((wave - half) * NACC + (a * V + t) * 8 + j) * kWave + lane] = make_float4(v[0], v[1], v[2], v[3]);
+                    }
         }
         __syncthreads();
         if (wave < half) {
 #pragma unroll
-            for (int t = 0; t < V; t++)
+            for (int a = 0; a < MS; a++)
 #pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const float4 v = red[(wave * NACC + t * 8 + j) * kWave + lane];
-                    y[t][j] += v4f{v.x, v.y, v.z, v.w};
-                }
+                for (int t = 0; t < V; t++)
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const float4 v = red[(wave * NACC + (a * V + t) * 8 + j) * kWave + lane];
+                        y[a][t][j] += v4f{v.x, v.y, v.z, v.w};
+                    }
         }
     }
     if (wave != 0 || !col_ok) return;
 
-    // ---- store: lane (word column li, quarter kb) holds tokens 4*kb + r for its 8*V channels -------
+    // ---- store: lane (word column li, quarter kb) holds tokens 16*a + 4*kb + r for its 8*V channels ---
     const bool split = gridDim.y > 1;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int m = 4 * kb + r;
-        if (m >= M) continue;
+    for (int a = 0; a < MS; a++) {
 #pragma unroll
-        for (int t = 0; t < V; t++) {
-            const int n = 8 * (cw + t);
-            if (split) {
-                float4* dst = reinterpret_cast<float4*>(partials + ((int64_t)blockIdx.y * M_total + m) * N + n);
-                dst[0] = make_float4(y[t][0][r], y[t][1][r], y[t][2][r], y[t][3][r]);
-                dst[1] = make_float4(y[t][4][r], y[t][5][r], y[t][6][r], y[t][7][r]);
-            } else {
-                uint32_t o[4];
+        for (int r = 0; r < 4; r++) {
+            const int m = 16 * a + 4 * kb + r;
+            if (m >= M) continue;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    float lo = y[t][2 * j][r], hi = y[t][2 * j + 1][r];
-                    if (bias) {
-                        lo = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(lo)) + Lo<LLMQ_F16>::to_f32(bias[n + 2 * j]);
-                        hi = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(hi)) + Lo<LLMQ_F16>::to_f32(bias[n + 2 * j + 1]);
+            for (int t = 0; t < V; t++) {
+                const int n = 8 * (cw + t);
+                if (split) {
+                    float4* dst = reinterpret_cast<float4*>(partials + ((int64_t)blockIdx.y * M_total + m) * N + n);
+                    dst[0] = make_float4(y[a][t][0][r], y[a][t][1][r], y[a][t][2][r], y[a][t][3][r]);
+                    dst[1] = make_float4(y[a][t][4][r], y[a][t][5][r], y[a][t][6][r], y[a][t][7][r]);
+                } else {
+                    uint32_t o[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float lo = y[a][t][2 * j][r], hi = y[a][t][2 * j + 1][r];
+                        if (bias) {
+                            lo = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(lo)) + Lo<LLMQ_F16>::to_f32(bias[n + 2 * j]);
+                            hi = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(hi)) + Lo<LLMQ_F16>::to_f32(bias[n + 2 * j + 1]);
+                        }
+                        o[j] = (uint32_t)Lo<LLMQ_F16>::from_f32(lo) | ((uint32_t)Lo<LLMQ_F16>::from_f32(hi) << 16);
                     }
-                    o[j] = (uint32_t)Lo<LLMQ_F16>::from_f32(lo) | ((uint32_t)Lo<LLMQ_F16>::from_f32(hi) << 16);
+                    *reinterpret_cast<uint4*>(out + (int64_t)m * N + n) = make_uint4(o[0], o[1], o[2], o[3]);
                 }
-                *reinterpret_cast<uint4*>(out + (int64_t)m * N + n) = make_uint4(o[0], o[1], o[2], o[3]);
             }
         }
     }
@@ -594,15 +661,24 @@ AwqPlan make_awq_plan(int64_t M, int64_t N, int64_t K) {
 
 // Decode kernel (group 128): a block = one column tile x one 16-token slab x KW wavefronts along K; a K split
 // across blocks only when the tiles alone cannot fill the GPU.
-struct DecodePlan { int v, kw, splits; };
-DecodePlan make_decode_plan(int64_t N, int64_t K) {
+struct DecodePlan { int v, kw, ms, splits; };
+DecodePlan make_decode_plan(int64_t M, int64_t N, int64_t K) {
     DecodePlan p;
     const int Nw = (int)(N / 8), groups = (int)(K / 128);
+    // Token tiles of 16 per wavefront.  Above 16 tokens, where the column tiles alone cannot fill the GPU
+    // (so that K is split across blocks anyway), one wavefront feeds every unpacked weight operand to 2 or 4
+    // token tiles instead of running one block per 16-token slab: measured at 64 tokens, down 41 -> 28 us,
+    // o 19 -> 18 us.  With many column tiles (gate_up) the slabs are as fast: every variant then spends its
+    // time re-reading the activations once per column tile.
+    p.ms = (cdiv(Nw, 16) < 128) ? (M > 32 ? 4 : (M > 16 ? 2 : 1)) : 1;
+    if (g_force_v == 5) p.ms = 2;
+    if (g_force_v == 6) p.ms = 4;
+    if (g_force_v == 1 || g_force_v == 2) p.ms = 1;
     // 128-byte row segments (V = 2) stream measurably faster than 64-byte ones; use them whenever
     // the tiles alone give every other CU a block, and then do without a second kernel.
-    p.v = (Nw % 2 == 0 && Nw / 32 >= 128) ? 2 : 1;
-    if (g_force_v == 1 || (g_force_v == 2 && Nw % 2 == 0)) p.v = g_force_v;
-    p.kw = (g_force_kw > 0 && p.v == 1) ? g_force_kw : 4;
+    p.v = (p.ms == 1 && Nw % 2 == 0 && Nw / 32 >= 128) ? 2 : 1;
+    if (p.ms == 1 && (g_force_v == 1 || (g_force_v == 2 && Nw % 2 == 0))) p.v = g_force_v;
+    p.kw = (g_force_kw > 0 && p.v == 1 && p.ms == 1) ? g_force_kw : 4;
     const int ntiles = cdiv(Nw, 16 * p.v);
     int splits = g_force_splits > 0 ? g_force_splits : (ntiles >= 128 ? 1 : cdiv(200, ntiles));  // measured optimum: ~200 blocks
     if (splits > groups / p.kw) splits = groups / p.kw;  // at least one group per wavefront
@@ -616,9 +692,9 @@ inline bool decode_path(int64_t M, int64_t group) { return M <= 64 && group == 1
 
 // More than 64 tokens go to the tile kernel (weights dequantized once per token tile on their way into LDS);
 // llmq_awq_force_plan(3 | 4, ...) forces its 64x128 | 256x256 tile for any M, (1 | 2, ...) keeps the slabs.
-inline bool tile_path(int64_t M) { return g_force_v >= 3 || (g_force_v == 0 && M > 64); }
+inline bool tile_path(int64_t M) { return g_force_v == 3 || g_force_v == 4 || (g_force_v == 0 && M > 64); }
 inline AwqTilePlan tile_plan(int64_t M, int64_t N, int64_t K) {
-    return make_awq_tile_plan(M, N, K, g_force_v >= 3 ? g_force_v - 3 : -1, g_force_splits);
+    return make_awq_tile_plan(M, N, K, (g_force_v == 3 || g_force_v == 4) ? g_force_v - 3 : -1, g_force_splits);
 }
 
 template <int V, int MT>
@@ -636,7 +712,7 @@ void launch_awq(const AwqPlan& p, const uint16_t* x, int64_t ldx, const uint32_t
 using namespace llmq;
 
 extern "C" int llmq_awq_force_plan(int v, int splits, int k_waves) {
-    if (v < 0 || v > 4 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
+    if (v < 0 || v > 6 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
     g_force_v = v;
     g_force_splits = splits;
     g_force_kw = k_waves;
@@ -655,7 +731,7 @@ extern "C" size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
         const AwqPlan p = make_awq_plan(mm, N, K);  // sized for either kernel (the group size is not known here)
         size_t need = p.splits > 1 ? (size_t)p.splits * mm * N * sizeof(float) : 0;
         if (K % 128 == 0) {
-            const DecodePlan d = make_decode_plan(N, K);
+            const DecodePlan d = make_decode_plan(mm, N, K);
             const size_t need2 = d.splits > 1 ? (size_t)d.splits * mm * N * sizeof(float) : 0;
             if (need2 > need) need = need2;
         }
@@ -704,17 +780,20 @@ extern "C" int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight,
         uint16_t* os = (uint16_t*)out + m0 * N;
         int splits;
         if (decode_path(mm, group)) {
-            const DecodePlan d = make_decode_plan(N, K);
+            const DecodePlan d = make_decode_plan(mm, N, K);
             splits = d.splits;
             if (splits > 1 && (!ws || workspace_bytes < (size_t)splits * mm * N * sizeof(float))) return LLMQ_ERR_WORKSPACE;
-            const int slabs = cdiv(mm, 16);
+            const int ms = d.ms;
+            const int slabs = cdiv(mm, 16 * ms);
             const dim3 grid(cdiv(Ni / 8, 16 * d.v) * slabs, splits);
-#define LLMQ_AWQ_DECODE(VV, KWW) \
-    hipLaunchKernelGGL((awq_gemv_kernel<VV, KWW>), grid, dim3(KWW * kWave), 0, st, xs, ldx, qw, sc, qz, bs, os, ws, mm, Ni, \
-                       Ki, slabs)
-            if (d.v == 2) LLMQ_AWQ_DECODE(2, 4);
-            else if (d.kw == 8) LLMQ_AWQ_DECODE(1, 8);
-            else LLMQ_AWQ_DECODE(1, 4);
+#define LLMQ_AWQ_DECODE(VV, KWW, MSS) \
+    hipLaunchKernelGGL((awq_gemv_kernel<VV, KWW, MSS>), grid, dim3(KWW * kWave), 0, st, xs, ldx, qw, sc, qz, bs, os, ws, mm, \
+                       Ni, Ki, slabs)
+            if (ms == 4) LLMQ_AWQ_DECODE(1, 4, 4);
+            else if (ms == 2) LLMQ_AWQ_DECODE(1, 4, 2);
+            else if (d.v == 2) LLMQ_AWQ_DECODE(2, 4, 1);
+            else if (d.kw == 8) LLMQ_AWQ_DECODE(1, 8, 1);
+            else LLMQ_AWQ_DECODE(1, 4, 1);
 #undef LLMQ_AWQ_DECODE
         } else {
             const AwqPlan p = make_awq_plan(mm, N, K);

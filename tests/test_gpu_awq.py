@@ -177,3 +177,23 @@ def test_tile_kernel_prefill_size(cuda):
     x = W.activations(M, K, 516, dtype=torch.float16, outliers=False)
     out = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8)
     assert rel_err(out, R.awq_gemm(x, qw, qz, s, 128)) <= REL_TOL
+
+
+@pytest.mark.parametrize("variant", [5, 6])
+@pytest.mark.parametrize("splits", [0, 2])
+@pytest.mark.parametrize("M,K,N", [(17, 1024, 264), (33, 512, 4608), (50, 3584, 1000), (64, 896, 4864), (3, 256, 136)])
+def test_streaming_kernel_with_shared_unpack(cuda, force_awq_plan, variant, splits, M, K, N):
+    """The streaming kernel with 2 (variant 5) or 4 (variant 6) token tiles per wavefront: every unpacked weight
+    operand feeds all tiles; weights are dequantized to fp16((q - z) * s) like the reference's."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    qw, qz, s = W.awq_weights(N, K, 11 * M + N)
+    x = W.activations(M, K, 12 * M + K, dtype=torch.float16, outliers=False)
+    bias = (0.1 * torch.randn(N, generator=torch.Generator().manual_seed(M))).half() if splits else None
+    ref = R.awq_gemm(x, qw, qz, s, 128)
+    if bias is not None:
+        ref = (ref.float() + bias.float()).half()
+    force_awq_plan(variant, splits)
+    out = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8,
+                          bias=None if bias is None else bias.to(cuda))
+    assert rel_err(out, ref) <= REL_TOL, (variant, splits, M, K, N)
