@@ -301,7 +301,12 @@ struct AwqTilePlan { int cfg, splits, k_per_split; };  // also declared in awq.h
 
 AwqTilePlan make_awq_tile_plan(int64_t M, int64_t N, int64_t K, int force_cfg, int force_splits) {
     AwqTilePlan p;
-    p.cfg = force_cfg >= 0 ? force_cfg : (M > 128 ? 1 : 0);
+    // The 256x256 tile needs enough tiles (or enough K per tile, when K is split) to fill the GPU; below
+    // that the 64x128 tile wins although it dequantizes every weight four times as often (measured on the
+    // Qwen2-7B shapes: 256x256 from 512 tokens for gate_up, from 1024 for down, never for qkv / o below 2048).
+    const int64_t tiles256 = (int64_t)cdiv(M, 256) * cdiv(N, 256);
+    const bool few_padding_rows = 4 * M >= 3 * (int64_t)cdiv(M, 256) * 256;
+    p.cfg = force_cfg >= 0 ? force_cfg : ((tiles256 * K >= (int64_t)224 * 3584 && few_padding_rows) ? 1 : 0);
     const int bm = p.cfg ? 256 : 64, bn = p.cfg ? 256 : 128;
     const int blocks = cdiv(M, bm) * cdiv(N, bn);
     const int want = p.cfg ? 256 : 512;  // blocks that fill the 256 CUs

@@ -22,13 +22,14 @@ def _pack_rows(values: torch.Tensor, w_bit: int = 4) -> torch.Tensor:
 
 
 def dequant_matmul_token_threshold(in_features: int) -> int:
-    """Token count from which dequantize + fp16 matmul beats the fused kernel on MI355X.
+    """Token count from which dequantize + fp16 matmul beats the fused kernels on MI355X.
 
-    The reference switches at 1024 tokens (linear_awq.py:22,47).  The fused kernel here streams the weights
-    once per 64 tokens, so its time grows with the token count while dequantize + matmul stays nearly flat:
-    measured crossovers on the Qwen2-7B shapes are ~180 tokens for K = 3584 (qkv, o, gate_up) and ~400 for
-    K = 18944 (down).  Both paths are within 1e-2 (max relative) of dequantize-then-matmul in fp32."""
-    return 192 if in_features <= 8192 else 384
+    The reference switches at 1024 tokens (linear_awq.py:22,47).  Measured on the Qwen2-7B shapes, the fused
+    path (streaming kernel up to 64 tokens, tile kernel with in-loop dequantization above) is ahead up to
+    ~400 tokens for K = 3584 (qkv, o, gate_up) and ~750 for K = 18944 (down); beyond that the dequantizer's
+    fixed cost is amortized and the library matmul runs at a higher rate than the tile kernel.  Both paths are
+    within 1e-2 (max relative) of dequantize-then-matmul in fp32."""
+    return 384 if in_features <= 8192 else 768
 
 
 def awq_linear_forward(x, qweight, qzeros, scales, w_bit=4, group_size=128, bias=None, out_features=0):
