@@ -665,19 +665,18 @@ struct DecodePlan { int v, kw, ms, splits; };
 DecodePlan make_decode_plan(int64_t M, int64_t N, int64_t K) {
     DecodePlan p;
     const int Nw = (int)(N / 8), groups = (int)(K / 128);
-    // Token tiles of 16 per wavefront.  Above 16 tokens, where the column tiles alone cannot fill the GPU
-    // (so that K is split across blocks anyway), one wavefront feeds every unpacked weight operand to 2 or 4
-    // token tiles instead of running one block per 16-token slab: measured at 64 tokens, down 41 -> 28 us,
-    // o 19 -> 18 us.  With many column tiles (gate_up) the slabs are as fast: every variant then spends its
-    // time re-reading the activations once per column tile.
-    p.ms = (cdiv(Nw, 16) < 128) ? (M > 32 ? 4 : (M > 16 ? 2 : 1)) : 1;
+    // Token tiles of 16 per wavefront.  Above 16 tokens, for a long K that is split across blocks anyway
+    // (down), one wavefront feeds every unpacked weight operand to 2 or 4 token tiles instead of running
+    // one block per 16-token slab: measured at 64 tokens with the weights coming from HBM, down 30.5 -> 27 us.
+    // For K = 3584 the slabs are as fast or faster (qkv 19 vs 21.6 us, gate_up 57 vs 65 us).
+    p.ms = (cdiv(Nw, 16) < 128 && K >= 8192) ? (M > 32 ? 4 : (M > 16 ? 2 : 1)) : 1;
     if (g_force_v == 5) p.ms = 2;
     if (g_force_v == 6) p.ms = 4;
     if (g_force_v == 1 || g_force_v == 2) p.ms = 1;
     // 128-byte row segments (V = 2) stream measurably faster than 64-byte ones; use them whenever
     // the tiles alone give every other CU a block, and then do without a second kernel.  With more than one
-    // 16-token slab per column tile the narrower tiles win: twice the blocks at two per CU instead of one
-    // pack the rounds better (gate_up at 64 tokens: 52 -> 43 us, at 32: 36 -> 29 us).
+    // 16-token slab per column tile the narrower tiles are slightly ahead: twice the blocks, two per CU
+    // instead of one (gate_up at 64 tokens: 58 -> 56.6 us from HBM, 52 -> 43 us with cache-resident weights).
     p.v = (p.ms == 1 && M <= 16 && Nw % 2 == 0 && Nw / 32 >= 128) ? 2 : 1;
     if (p.ms == 1 && (g_force_v == 1 || (g_force_v == 2 && Nw % 2 == 0))) p.v = g_force_v;
     p.kw = (g_force_kw > 0 && p.v == 1 && p.ms == 1) ? g_force_kw : 4;
