@@ -693,9 +693,9 @@ inline bool decode_path(int64_t M, int64_t group) { return M <= 64 && group == 1
 
 // More than 64 tokens go to the tile kernel (weights dequantized once per token tile on their way into LDS);
 // llmq_awq_force_plan(3 | 4, ...) forces its 64x128 | 256x256 tile for any M, (1 | 2, ...) keeps the slabs.
-inline bool tile_path(int64_t M) { return g_force_v == 3 || g_force_v == 4 || (g_force_v == 0 && M > 64); }
+inline bool tile_path(int64_t M) { return g_force_v == 3 || g_force_v == 4 || g_force_v == 7 || (g_force_v == 0 && M > 64); }
 inline AwqTilePlan tile_plan(int64_t M, int64_t N, int64_t K) {
-    return make_awq_tile_plan(M, N, K, (g_force_v == 3 || g_force_v == 4) ? g_force_v - 3 : -1, g_force_splits);
+    return make_awq_tile_plan(M, N, K, (g_force_v == 3 || g_force_v == 4) ? g_force_v - 3 : (g_force_v == 7 ? 2 : -1), g_force_splits);
 }
 
 template <int V, int MT>
@@ -713,7 +713,7 @@ void launch_awq(const AwqPlan& p, const uint16_t* x, int64_t ldx, const uint32_t
 using namespace llmq;
 
 extern "C" int llmq_awq_force_plan(int v, int splits, int k_waves) {
-    if (v < 0 || v > 6 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
+    if (v < 0 || v > 7 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
     g_force_v = v;
     g_force_splits = splits;
     g_force_kw = k_waves;

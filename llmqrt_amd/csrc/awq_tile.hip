@@ -296,20 +296,25 @@ int launch_tile(const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16
 
 }  // namespace
 
-// Tile shapes: 0 = 64 tokens x 128 channels (4 wavefronts), 1 = 256 x 256 (8 wavefronts).
+// Tile shapes: 0 = 64 tokens x 128 channels (4 wavefronts), 1 = 256 x 256 (8 wavefronts), 2 = 128 x 128 (4 wavefronts).
 struct AwqTilePlan { int cfg, splits, k_per_split; };  // also declared in awq.hip
 
 AwqTilePlan make_awq_tile_plan(int64_t M, int64_t N, int64_t K, int force_cfg, int force_splits) {
     AwqTilePlan p;
-    // The 256x256 tile needs enough tiles (or enough K per tile, when K is split) to fill the GPU; below
-    // that the 64x128 tile wins although it dequantizes every weight four times as often (measured on the
-    // Qwen2-7B shapes: 256x256 from 512 tokens for gate_up, from 1024 for down, never for qkv / o below 2048).
-    const int64_t tiles256 = (int64_t)cdiv(M, 256) * cdiv(N, 256);
-    const bool few_padding_rows = 4 * M >= 3 * (int64_t)cdiv(M, 256) * 256;
-    p.cfg = force_cfg >= 0 ? force_cfg : ((tiles256 * K >= (int64_t)224 * 3584 && few_padding_rows) ? 1 : 0);
-    const int bm = p.cfg ? 256 : 64, bn = p.cfg ? 256 : 128;
+    // Modelled cost = token rows after padding to the tile height x a per-row cost measured on the Qwen2-7B
+    // shapes (the larger the tile, the fewer times a weight is dequantized and the fewer LDS bytes per MAC),
+    // for the tiles that can fill the GPU: 256x256 needs 400 tiles, 128x128 needs 256 blocks' worth of work
+    // (weighted by K, since a long K is split across blocks at little cost).
+    const int64_t pad64 = (int64_t)cdiv(M, 64) * 64, pad128 = (int64_t)cdiv(M, 128) * 128, pad256 = (int64_t)cdiv(M, 256) * 256;
+    const int64_t tiles256 = (int64_t)cdiv(M, 256) * cdiv(N, 256), blocks128 = (int64_t)cdiv(M, 128) * cdiv(N, 128);
+    const double cost64 = (double)pad64;
+    const double cost128 = blocks128 * K >= (int64_t)256 * 3584 ? 0.85 * pad128 : 1e30;
+    const double cost256 = tiles256 >= 400 ? 0.72 * pad256 : 1e30;
+    p.cfg = cost256 <= cost128 && cost256 <= cost64 ? 1 : (cost128 <= cost64 ? 2 : 0);
+    if (force_cfg >= 0) p.cfg = force_cfg;
+    const int bm = p.cfg == 1 ? 256 : (p.cfg == 2 ? 128 : 64), bn = p.cfg == 1 ? 256 : 128;
     const int blocks = cdiv(M, bm) * cdiv(N, bn);
-    const int want = p.cfg ? 256 : 512;  // blocks that fill the 256 CUs
+    const int want = p.cfg == 1 ? 256 : 512;  // blocks that fill the 256 CUs
     int splits = force_splits > 0 ? force_splits : (blocks >= want * 3 / 4 ? 1 : cdiv(want, blocks));
     const int max_splits = (int)(K / 256) > 0 ? (int)(K / 256) : 1;  // at least 4 K tiles per block
     if (splits > max_splits) splits = max_splits;
@@ -322,7 +327,8 @@ AwqTilePlan make_awq_tile_plan(int64_t M, int64_t N, int64_t K, int force_cfg, i
 int launch_awq_tile(const AwqTilePlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
                     const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K, int G,
                     hipStream_t st) {
-    if (p.cfg) return launch_tile<TileCfg<256, 256, 2, 4>>(x, ldx, qw, scales, qz, bias, out, ws, M, N, K, G, p.splits, p.k_per_split, st);
+    if (p.cfg == 2) return launch_tile<TileCfg<128, 128, 2, 2>>(x, ldx, qw, scales, qz, bias, out, ws, M, N, K, G, p.splits, p.k_per_split, st);
+    if (p.cfg == 1) return launch_tile<TileCfg<256, 256, 2, 4>>(x, ldx, qw, scales, qz, bias, out, ws, M, N, K, G, p.splits, p.k_per_split, st);
     return launch_tile<TileCfg<64, 128, 1, 4>>(x, ldx, qw, scales, qz, bias, out, ws, M, N, K, G, p.splits, p.k_per_split, st);
 }
 

@@ -26,10 +26,10 @@ def dequant_matmul_token_threshold(in_features: int) -> int:
 
     The reference switches at 1024 tokens (linear_awq.py:22,47).  Measured on the Qwen2-7B shapes, the fused
     path (streaming kernel up to 64 tokens, tile kernel with in-loop dequantization above) is ahead up to
-    ~400 tokens for K = 3584 (qkv, o, gate_up) and ~750 for K = 18944 (down); beyond that the dequantizer's
+    ~400 (qkv) to ~560 (gate_up) tokens for K = 3584 and ~900 for K = 18944 (down); beyond that the dequantizer's
     fixed cost is amortized and the library matmul runs at a higher rate than the tile kernel.  Both paths are
     within 1e-2 (max relative) of dequantize-then-matmul in fp32."""
-    return 384 if in_features <= 8192 else 768
+    return 448 if in_features <= 8192 else 896
 
 
 def awq_linear_forward(x, qweight, qzeros, scales, w_bit=4, group_size=128, bias=None, out_features=0):

@@ -144,11 +144,11 @@ TILE_SHAPES = [(300, 1056, 520, 32), (65, 64, 8, 64), (1, 96, 136, 32), (257, 51
                (64, 1024, 1000, 128)]
 
 
-@pytest.mark.parametrize("tile", [3, 4])
+@pytest.mark.parametrize("tile", [3, 4, 7])
 @pytest.mark.parametrize("splits", [0, 1, 3])
 @pytest.mark.parametrize("M,K,N,G", TILE_SHAPES)
 def test_tile_kernel_every_shape_and_split(cuda, force_awq_plan, tile, splits, M, K, N, G):
-    """The many-token tile kernel (both tile shapes, fused and split-K) against the oracle.  Its weights are
+    """The many-token tile kernel (all three tile shapes, fused and split-K) against the oracle.  Its weights are
     fp16((q - z) * s) as in the reference dequantizer, accumulated in fp32."""
     from llmqrt_amd import workloads as W
     from llmqrt_amd.awq_kernels import awq_gemm_triton
