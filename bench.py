@@ -51,6 +51,9 @@ def parse_args():
     ap.add_argument("--awq-only", action="store_true",
                     help="profiler mode: only the W4A16 launches of configs[3] (4 projections x M in {1,4,16,64}), "
                          "weights rotated beyond the Infinity Cache, preceded by one 256 MiB calibration copy")
+    ap.add_argument("--awq-prefill-only", action="store_true",
+                    help="profiler mode: only the W4A16 tile kernel (4 projections x M in {128,256,512,2048}), "
+                         "preceded by one 256 MiB calibration copy")
     ap.add_argument("--quant-only", action="store_true",
                     help="profiler mode: only the row kernels (int8 / fp8 per-token quantizers, RMSNorm, RMSNorm fused "
                          "with the int8 quantizer) at M in {2048, 8192} x K in {3584, 18944}, after one 256 MiB copy")
@@ -255,8 +258,23 @@ def details_awq(dev):
             dequant()
             torch.matmul(xp, deq)
         t_pre = batch_time_us([prefill], stream_obj, 10)
+        mid = {}
+        for Mm in (256, 512):
+            xm = W.activations(Mm, K, W.seed_for(3, 950 + pi + Mm), dtype=torch.float16, outliers=False).to(dev)
+            om = torch.empty((Mm, N), dtype=torch.float16, device=dev)
+            wsm = torch.empty(max(L.llmq_awq_gemm_workspace_bytes(Mm, N, K), 16), dtype=torch.uint8, device=dev)
+
+            def fused():
+                L.llmq_awq_gemm(xm.data_ptr(), K, c[0].data_ptr(), c[2].data_ptr(), c[1].data_ptr(), None, om.data_ptr(),
+                                Mm, N, K, 128, wsm.data_ptr(), wsm.numel(), stream)
+
+            def unfused():
+                dequant()
+                torch.matmul(xm, deq)
+            mid[f"M{Mm}_tile_kernel_us"] = round(batch_time_us([fused], stream_obj, 20), 1)
+            mid[f"M{Mm}_dequant_plus_fp16_matmul_us"] = round(batch_time_us([unfused], stream_obj, 20), 1)
         db = K * N // 2 + 2 * K * N
-        rows.append({"proj": pname, "dequant_us": round(t_deq, 2), "dequant_GBs": round(db / t_deq / 1e3, 1),
+        rows.append({"proj": pname, **mid, "dequant_us": round(t_deq, 2), "dequant_GBs": round(db / t_deq / 1e3, 1),
                      "dequant_pct_hbm_peak": round(100 * db / t_deq / 1e3 / PEAK_HBM_GBS, 2),
                      "prefill_M2048_dequant_plus_fp16_matmul_us": round(t_pre, 1),
                      "prefill_M2048_TFLOPs": round(2 * 2048 * N * K / t_pre / 1e6, 1)})
@@ -294,6 +312,38 @@ def awq_only(dev, steps, warmup):
             assert rc == 0
     torch.cuda.synchronize()
     print(json.dumps({"awq_only": True, "order": order, "steps": steps, "warmup": warmup,
+                      "calibration_copy_bytes_each_way": cal_src.numel() * 4}))
+
+
+AWQ_PREFILL_M = (128, 256, 512, 2048)
+
+
+def awq_prefill_only(dev, steps, warmup):
+    """For profiler runs: the W4A16 tile kernel (more than 64 tokens) on the four projections, after one plain
+    copy of known size that calibrates the HBM byte counters."""
+    from llmqrt_amd import _abi, workloads as W
+    L = _abi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    cal_src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    launches, order = [], []
+    for pi, (pname, (K, N)) in enumerate(W.QWEN2_7B_PROJ.items()):
+        qw, qz, sc = (t.to(dev) for t in W.awq_weights(N, K, W.seed_for(3, 100 + pi)))
+        for mi, M in enumerate(AWQ_PREFILL_M):
+            x = W.activations(M, K, W.seed_for(3, 50 * pi + mi), dtype=torch.float16, outliers=False).to(dev)
+            out = torch.empty((M, N), dtype=torch.float16, device=dev)
+            wsp = torch.empty(max(L.llmq_awq_gemm_workspace_bytes(M, N, K), 16), dtype=torch.uint8, device=dev)
+            launches.append((x, out, wsp, (qw, qz, sc), M, N, K))
+            order.append(f"{pname}_M{M}")
+    torch.cuda.synchronize()
+    for it in range(warmup + steps):
+        for (x, out, wsp, c, M, N, K) in launches:
+            rc = L.llmq_awq_gemm(x.data_ptr(), K, c[0].data_ptr(), c[2].data_ptr(), c[1].data_ptr(), None, out.data_ptr(),
+                                 M, N, K, 128, wsp.data_ptr(), wsp.numel(), stream)
+            assert rc == 0
+    torch.cuda.synchronize()
+    print(json.dumps({"awq_prefill_only": True, "order": order, "steps": steps, "warmup": warmup,
                       "calibration_copy_bytes_each_way": cal_src.numel() * 4}))
 
 
@@ -440,6 +490,9 @@ def main():
 
     if args.awq_only:
         awq_only(dev, args.steps, args.warmup)
+        return
+    if args.awq_prefill_only:
+        awq_prefill_only(dev, args.steps, args.warmup)
         return
     if args.quant_only:
         quant_only(dev, args.steps, args.warmup)
