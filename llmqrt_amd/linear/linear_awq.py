@@ -21,6 +21,11 @@ def _pack_rows(values: torch.Tensor, w_bit: int = 4) -> torch.Tensor:
     return torch.where(word >= 2 ** 31, word - 2 ** 32, word).to(torch.int32)
 
 
+# Set to False to keep every token count on this package's own kernels (llmq_awq_gemm) instead of switching to
+# dequantize + torch.matmul for long prompts.
+USE_DEQUANT_MATMUL = True
+
+
 def dequant_matmul_token_threshold(in_features: int) -> int:
     """Token count from which dequantize + fp16 matmul beats the fused kernels on MI355X.
 
@@ -38,7 +43,7 @@ def awq_linear_forward(x, qweight, qzeros, scales, w_bit=4, group_size=128, bias
     if x.shape[0] == 0:
         return torch.zeros(out_shape, dtype=x.dtype, device=x.device)
     tokens = x.numel() // x.shape[-1]
-    if tokens >= dequant_matmul_token_threshold(x.shape[-1]):
+    if USE_DEQUANT_MATMUL and tokens >= dequant_matmul_token_threshold(x.shape[-1]):
         w = awq_dequantize_triton(qweight, scales, qzeros)
         out = torch.matmul(x, w.to(x.dtype))
         out = out + bias if bias is not None else out

@@ -129,6 +129,14 @@ def test_module_paths_agree_around_the_token_threshold(cuda, K):
         y = m(x.to(cuda).view(1, M, K))
         assert y.shape == (1, M, N) and y.dtype == torch.float16
         assert rel_err(y.view(M, N), R.awq_gemm(x, qw, qz, sc, 128)) <= REL_TOL
+    # with the switch off the same token count stays on the fused kernels
+    from llmqrt_amd.linear import linear_awq
+    linear_awq.USE_DEQUANT_MATMUL = False
+    try:
+        y2 = m(x.to(cuda).view(1, t, K))
+    finally:
+        linear_awq.USE_DEQUANT_MATMUL = True
+    assert rel_err(y2.view(t, N), R.awq_gemm(x, qw, qz, sc, 128)) <= REL_TOL
 
 
 @pytest.fixture
