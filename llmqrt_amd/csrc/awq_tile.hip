@@ -88,12 +88,14 @@ __global__ __launch_bounds__(C::NT) void awq_tile_kernel(
     constexpr int ROWS_STEP = C::NT / kCPR;
     const int ld_row = tid / kCPR, ld_c = tid % kCPR;
     const uint16_t* a_base = x + (int64_t)m0 * ldx + k_begin;
-    int a_off[C::A_LOADS], st_a[C::A_LOADS];
-#pragma unroll
-    for (int i = 0; i < C::A_LOADS; i++) {
-        a_off[i] = min(ld_row + i * ROWS_STEP, M - 1 - m0) * (int)ldx;
-        st_a[i] = lds_chunk(ld_row + i * ROWS_STEP, ld_c);
-    }
+    // Row offsets and LDS slots are recomputed per use instead of kept in registers (the 256x256 tile has
+    // none to spare); with a row step that is a multiple of 64 the xor term of the slot is the same for all i.
+    const int last_row = M - 1 - m0;
+    auto a_off = [&](int i) { return min(ld_row + i * ROWS_STEP, last_row) * (int)ldx; };
+    const int st_a0 = lds_chunk(ld_row, ld_c);
+    auto st_a = [&](int i) {
+        return (ROWS_STEP % 64 == 0) ? st_a0 + i * ROWS_STEP * kCPR : lds_chunk(ld_row + i * ROWS_STEP, ld_c);
+    };
 
     // ---- weights: thread = (word column wc, channel half wh, k octet wo) ---------------------------
     const int wc = tid % C::WORDS, wh = (tid / C::WORDS) & 1, wo = tid / (2 * C::WORDS);
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(C::NT) void awq_tile_kernel(
         const int ktc = max(min(kt, ktiles - 1), 0) * kBK;
         const int ka = min(ktc + ld_c * 8, klen - 8);
 #pragma unroll
-        for (int i = 0; i < C::A_LOADS; i++) a_reg[i] = *reinterpret_cast<const uint4*>(a_base + a_off[i] + ka);
+        for (int i = 0; i < C::A_LOADS; i++) a_reg[i] = *reinterpret_cast<const uint4*>(a_base + a_off(i) + ka);
         const int kw = k_begin + min(ktc + wo * 8, klen - 8);
         const uint32_t* wp = qw + (int64_t)kw * Nw + cw;
 #pragma unroll
@@ -124,7 +126,7 @@ __global__ __launch_bounds__(C::NT) void awq_tile_kernel(
 #pragma unroll
         for (int i = 0; i < C::A_LOADS; i++) {
             const uint4 v = a_reg[i];
-            sA[st_a[i]] = make_uint4(v.x & keep_a, v.y & keep_a, v.z & keep_a, v.w & keep_a);
+            sA[st_a(i)] = make_uint4(v.x & keep_a, v.y & keep_a, v.z & keep_a, v.w & keep_a);
         }
         const uint32_t keep_w = (kt < ktiles && kt * kBK + wo * 8 < klen) ? 0xffffffffu : 0u;
         const uint32_t sw[4] = {s_reg.x, s_reg.y, s_reg.z, s_reg.w};
