@@ -34,7 +34,7 @@ if ROOT not in sys.path:
 # WRITE_SIZE of two `rocprofv3 --pmc` runs of `bench.py --roofline-only`, each scaled by what the same
 # counter reads for the 256 MiB calibration copy (2.000 and 1.000); see
 # profiles/gemm_w8a8_int8_mfma_prefill_qwen2_7b.md.  A measured constant: counters cannot be read from here.
-ROOFLINE_TRAFFIC_BYTES = 665222820
+ROOFLINE_TRAFFIC_BYTES = 628724706
 CPU_BASELINE_REPS = 12        # bounded CPU sample: about 10-15 s of host work
 PEAK_INT8_TOPS = 5033.0   # dense int8 MFMA peak of MI355X, TOP/s (256 CU x 2.4 GHz x 8192 op/clk)
 PEAK_FP8_TFLOPS = 5033.0  # dense fp8 MFMA peak

@@ -23,6 +23,10 @@
 
 #include "llmq_common.h"
 
+#ifndef LLMQ_LDS_EPILOGUE
+#define LLMQ_LDS_EPILOGUE 1
+#endif
+
 namespace llmq {
 namespace {
 
@@ -342,6 +346,73 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
         (reinterpret_cast<uintptr_t>(ep.w_scale) & 15u) == 0) {
         auto fast = [&](auto out_dt_c) {
             constexpr int ODT = decltype(out_dt_c)::value;
+            // Wave tiles of 64 channels: transpose through LDS (8 KB per wavefront, 64 token rows at a time) so
+            // that a store instruction writes 8 whole 128-byte rows instead of 32 pieces of 32 bytes.
+            constexpr bool LDS_EPI = LLMQ_LDS_EPILOGUE && C::TM % 2 == 0 && C::TN == 2 && C::LDS_BYTES >= (C::NT / kWave) * 8192u;
+            if constexpr (LDS_EPI) {
+                __syncthreads();  // every wavefront is done reading the operand stages
+                uint4* region = lds + wave * 512;
+#pragma unroll
+                for (int p = 0; p < C::TM / 2; p++) {
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        // scales and bias of this 32-channel tile (re-read per pass: they sit in L1, and keeping
+                        // both tiles' worth in registers would not fit beside the accumulators)
+                        float sw[16], bb[16];
+#pragma unroll
+                        for (int g = 0; g < 4; g++) {
+                            const int n = n0 + wn * C::WTN + j * 32 + 8 * g + 4 * khalf;
+                            if (ep.w_scale) {
+                                const float4 v = *reinterpret_cast<const float4*>(ep.w_scale + n);
+                                sw[4 * g] = v.x, sw[4 * g + 1] = v.y, sw[4 * g + 2] = v.z, sw[4 * g + 3] = v.w;
+                            } else {
+                                sw[4 * g] = sw[4 * g + 1] = sw[4 * g + 2] = sw[4 * g + 3] = 1.f;
+                            }
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                bb[4 * g + e] = ep.bias ? ep.beta * load_as_f32(ep.bias, ep.bias_dtype, n + e) : 0.f;
+                        }
+#pragma unroll
+                        for (int ii = 0; ii < 2; ii++) {
+                            const int i = 2 * p + ii;
+                            const int m = m0 + wm * C::WTM + i * 32 + l32;
+                            const float sa = ep.a_scale ? ep.a_scale[m] : 1.f;
+                            const int row = ii * 32 + l32, swz = (row >> 1) & 7;
+                            uint32_t pk[4][2];
+#pragma unroll
+                            for (int g = 0; g < 4; g++) {
+                                uint16_t h[4];
+#pragma unroll
+                                for (int e = 0; e < 4; e++) {
+                                    const auto av = acc[i][j][4 * g + e];
+                                    h[e] = Lo<ODT>::from_f32(epi_value((float)av, sa, sw[4 * g + e], alpha, bb[4 * g + e]));
+                                }
+                                pk[g][0] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+                                pk[g][1] = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+                            }
+#pragma unroll
+                            for (int g = 0; g < 2; g++) {
+#pragma unroll
+                                for (int x = 0; x < 2; x++) {
+                                    const auto sw2 = __builtin_amdgcn_permlane32_swap(pk[2 * g][x], pk[2 * g + 1][x], false, false);
+                                    pk[2 * g][x] = sw2[0];
+                                    pk[2 * g + 1][x] = sw2[1];
+                                }
+                                const int chunk = 4 * j + 2 * g + khalf;  // 8 channels = 16 bytes
+                                region[row * 8 + (chunk ^ swz)] = make_uint4(pk[2 * g][0], pk[2 * g][1], pk[2 * g + 1][0], pk[2 * g + 1][1]);
+                            }
+                        }
+                    }
+                    uint16_t* obase = reinterpret_cast<uint16_t*>(out) + (int64_t)(m0 + wm * C::WTM + p * 64) * ldo + n0 + wn * C::WTN;
+#pragma unroll
+                    for (int it = 0; it < 8; it++) {
+                        const int q = it * kWave + lane, row = q >> 3, c = q & 7;
+                        const uint4 v = region[row * 8 + (c ^ ((row >> 1) & 7))];
+                        *reinterpret_cast<uint4*>(obase + (int64_t)row * ldo + 8 * c) = v;
+                    }
+                }
+                return;
+            }
 #pragma unroll
             for (int j = 0; j < C::TN; j++) {
                 const int nb = n0 + wn * C::WTN + j * 32;
