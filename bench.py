@@ -35,6 +35,10 @@ if ROOT not in sys.path:
 # counter reads for the 256 MiB calibration copy (2.000 and 1.000); see
 # profiles/gemm_w8a8_int8_mfma_prefill_qwen2_7b.md.  A measured constant: counters cannot be read from here.
 ROOFLINE_TRAFFIC_BYTES = 628724706
+# The same for the FP8 launches (bench.py --fp8-only, profiles/gemm_fp8_mfma_prefill_qwen2_7b.md) and the W4A16
+# decode launches at M <= 16 (bench.py --awq-only, profiles/awq_gemv_w4a16_decode_qwen2_7b.md); None = not measured.
+FP8_TRAFFIC_BYTES = None
+W4A16_TRAFFIC_BYTES = None
 CPU_BASELINE_REPS = 12        # bounded CPU sample: about 10-15 s of host work
 PEAK_INT8_TOPS = 5033.0   # dense int8 MFMA peak of MI355X, TOP/s (256 CU x 2.4 GHz x 8192 op/clk)
 PEAK_FP8_TFLOPS = 5033.0  # dense fp8 MFMA peak
@@ -57,6 +61,9 @@ def parse_args():
     ap.add_argument("--quant-only", action="store_true",
                     help="profiler mode: only the row kernels (int8 / fp8 per-token quantizers, RMSNorm, RMSNorm fused "
                          "with the int8 quantizer) at M in {2048, 8192} x K in {3584, 18944}, after one 256 MiB copy")
+    ap.add_argument("--fp8-only", action="store_true",
+                    help="profiler mode: only the FP8 GEMM launches (4 projections x M in {512, 4096}), preceded by "
+                         "one 256 MiB calibration copy")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant kernel's launches (for rocprofv3 summaries)")
     return ap.parse_args()
@@ -65,10 +72,11 @@ def parse_args():
 class W8A8Linear:
     """One W8A8 linear with preallocated buffers; launch() = quantizer + GEMM through the C ABI."""
 
-    def __init__(self, name, M, K, N, qweight, w_scale, seed, dev):
+    def __init__(self, name, M, K, N, qweight, w_scale, seed, dev, x=None, norm_weight=None, eps=1e-6):
         from llmqrt_amd import _abi, workloads as W
         self.name, self.M, self.K, self.N = name, M, K, N
-        self.x = W.activations(M, K, seed).to(dev)
+        self.x = (W.activations(M, K, seed) if x is None else x).to(dev)
+        self.norm_weight, self.eps = norm_weight, eps   # set: RMSNorm fused into the quantizer launch
         self.qweight, self.w_scale = qweight, w_scale
         self.qx = torch.empty((M, K), dtype=torch.int8, device=dev)
         self.a_scale = torch.empty((M,), dtype=torch.float32, device=dev)
@@ -81,6 +89,11 @@ class W8A8Linear:
         self.ops = 2 * M * N * K
 
     def quant(self, stream):
+        if self.norm_weight is not None:
+            return self.L.llmq_rmsnorm_quant_i8_per_token(self.x.data_ptr(), self.abi.BF16, self.M, self.K, self.K,
+                                                          self.norm_weight.data_ptr(), self.eps, None,
+                                                          self.qx.data_ptr(), self.a_scale.data_ptr(), self.abi.F32,
+                                                          None, stream)
         return self.L.llmq_quant_i8_per_token(self.x.data_ptr(), self.abi.BF16, self.M, self.K, self.K,
                                               self.qx.data_ptr(), self.a_scale.data_ptr(), self.abi.F32, stream)
 
@@ -216,7 +229,76 @@ def details_fp8(dev):
     return rows
 
 
-def details_awq(dev):
+FP8_PREFILL_M = (512, 4096)
+
+
+def fp8_only(dev, steps, warmup):
+    """For profiler runs: the FP8 GEMM launches at the prefill sizes of configs[2] in a fixed order, after one
+    plain copy of known size that calibrates the HBM byte counters."""
+    from llmqrt_amd import _abi, workloads as W
+    L = _abi.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    cal_src = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
+    cal_dst = torch.empty_like(cal_src)
+    launches, order = [], []
+    for pi, (pname, (K, N)) in enumerate(W.QWEN2_7B_PROJ.items()):
+        wq, ws = (t.to(dev) for t in W.fp8_weights(N, K, W.seed_for(2, 100 + pi)))
+        for M in FP8_PREFILL_M:
+            mi = W.FP8_M.index(M)
+            x = W.activations(M, K, W.seed_for(2, 10 * pi + mi)).to(dev)
+            xq = torch.empty((M, K), dtype=torch.float8_e4m3fn, device=dev)
+            xs = torch.empty((M,), dtype=torch.float32, device=dev)
+            out = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+            wsp = torch.empty(max(L.llmq_gemm_workspace_bytes(M, N, K), 16), dtype=torch.uint8, device=dev)
+            assert L.llmq_quant_fp8_per_token(x.data_ptr(), _abi.BF16, M, K, K, xq.data_ptr(), xs.data_ptr(), stream) == 0
+            launches.append((xq, xs, wq, ws, out, wsp, M, N, K))
+            order.append(f"{pname}_M{M}")
+    torch.cuda.synchronize()
+    cal_dst.copy_(cal_src)
+    for it in range(warmup + steps):
+        for (xq, xs, wq, ws, out, wsp, M, N, K) in launches:
+            rc = L.llmq_gemm_fp8(xq.data_ptr(), _abi.E4M3, K, wq.data_ptr(), K, xs.data_ptr(), ws.data_ptr(), 1.0, None,
+                                 None, 0, 0.0, out.data_ptr(), _abi.BF16, N, M, N, K, None, wsp.data_ptr(), wsp.numel(),
+                                 stream)
+            assert rc == 0
+        if it + 1 == warmup:
+            torch.cuda.synchronize()
+    torch.cuda.synchronize()
+    print(json.dumps({"fp8_only": True, "order": order, "steps": steps, "warmup": warmup,
+                      "calibration_copy_bytes_each_way": cal_src.numel() * 4}))
+
+
+def roofline_fp8(rows):
+    """FP8 GEMM at the prefill sizes (M >= 512) of configs[2]: sum(2MNK) over the sum of the launch times."""
+    from llmqrt_amd import workloads as W
+    sel = [r for r in rows if r["M"] >= 512]
+    ops = sum(2 * r["M"] * W.QWEN2_7B_PROJ[r["proj"]][1] * W.QWEN2_7B_PROJ[r["proj"]][0] for r in sel)
+    us = sum(r["gemm_us"] for r in sel)
+    alg = sum(W.w8a8_gemm_bytes(r["M"], W.QWEN2_7B_PROJ[r["proj"]][1], W.QWEN2_7B_PROJ[r["proj"]][0]) for r in sel)
+    ach = ops / us / 1e6
+    return {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(ach / PEAK_FP8_TFLOPS, 4), "traffic": FP8_TRAFFIC_BYTES,
+            "algorithmic_bytes": alg // len(sel),
+            "kernel": "gemm_tile_kernel<fp8 e4m3> at M in {512, 4096} x {qkv, o, gate_up, down}",
+            "avg_launch_us": round(us / len(sel), 2)}
+
+
+def roofline_w4a16(rows):
+    """AWQ W4A16 decode (M <= 16) of configs[3], weights streamed from HBM (rotated beyond the Infinity Cache):
+    sum of algorithmic bytes over the sum of the launch times."""
+    from llmqrt_amd import workloads as W
+    sel = [r for r in rows if "M" in r and r["M"] <= 16]
+    b = sum(W.awq_gemm_bytes(r["M"], W.QWEN2_7B_PROJ[r["proj"]][1], W.QWEN2_7B_PROJ[r["proj"]][0]) for r in sel)
+    us = sum(r["us_hbm"] for r in sel)
+    ach = b / us / 1e3
+    return {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": W4A16_TRAFFIC_BYTES,
+            "algorithmic_bytes": b // len(sel),
+            "kernel": "AWQ decode kernels behind llmq_awq_gemm at M in {1, 4, 16} x {qkv, o, gate_up, down}",
+            "avg_launch_us": round(us / len(sel), 2)}
+
+
+def details_awq(dev, full=True):
     from llmqrt_amd import _abi, workloads as W
     L = _abi.lib()
     stream_obj = torch.cuda.current_stream()
@@ -245,6 +327,9 @@ def details_awq(dev):
             rows.append({"proj": pname, "M": M, "us_hbm": round(t_rot, 2), "us_cache_resident": round(t_res, 2),
                          "GBs_hbm": round(b / t_rot / 1e3, 1), "pct_hbm_peak": round(100 * b / t_rot / 1e3 / PEAK_HBM_GBS, 2),
                          "GBs_cache_resident": round(b / t_res / 1e3, 1), "weight_copies_rotated": ncopies})
+        if not full:
+            del copies
+            continue
         # prefill side of the module: the dequantizer (weights resident), alone and followed by the fp16 matmul
         deq = torch.empty((K, N), dtype=torch.float16, device=dev)
         c = copies[0]
@@ -381,28 +466,24 @@ def quant_only(dev, steps, warmup):
 
 def details_layer(dev):
     """Config 4: one decoder layer's linears (qkv, o, gate_up, down) in W8A8 with SmoothQuant factors
-    (alpha = 0.5) folded into the preceding norm weight / the weights; prefill 2048 tokens and decode 32."""
+    (alpha = 0.5) folded into the preceding RMSNorm weight (qkv, gate_up: one fused RMSNorm + per-token
+    quantizer launch on the residual stream) or into the producer's weights (o, down: their inputs arrive
+    divided by s; plain per-token quantizer); prefill 2048 tokens and decode 32.  The same tensors and launches
+    are checked against the oracle in tests/test_gpu_layer_stack.py."""
     from llmqrt_amd import _abi, workloads as W
     stream_obj = torch.cuda.current_stream()
     stream = stream_obj.cuda_stream
     out = []
-    projs = list(W.QWEN2_7B_PROJ.items())
-    weights = {}
-    for pi, (pname, (K, N)) in enumerate(projs):
-        w = W.dense_weights(N, K, W.seed_for(4, 100 + pi))
-        calib = W.activations(256, K, W.seed_for(4, 200 + pi)).float()
-        s = W.smoothquant_factors(calib.abs().amax(0), w.abs().amax(0), 0.5)
-        ws = w * s.view(1, -1)                                   # weights absorb s
-        scale = ws.abs().amax(dim=1) / 127
-        qw = (ws / scale.view(-1, 1)).round().clamp(-128, 127).to(torch.int8)
-        weights[pname] = (qw.to(dev), scale.to(dev), s)
-    for M in (2048, 32):
+    layer = W.smoothquant_layer(alpha=0.5)
+    dev_w = {n: (p["qweight"].to(dev), p["w_scale"].to(dev),
+                 None if p["norm_weight_folded"] is None else p["norm_weight_folded"].to(dev))
+             for n, p in layer.items()}
+    for M in W.LAYER_M:
         lins = []
-        for pi, (pname, (K, N)) in enumerate(projs):
-            qw, scale, s = weights[pname]
-            lin = W8A8Linear(f"{pname}_M{M}", M, K, N, qw, scale, W.seed_for(4, 10 * pi), dev)
-            lin.x = (lin.x.float().cpu() / s.view(1, -1)).bfloat16().to(dev)   # activations arrive pre-divided by s
-            lins.append(lin)
+        for pname, p in layer.items():
+            qw, scale, gf = dev_w[pname]
+            lins.append(W8A8Linear(f"{pname}_M{M}", M, p["K"], p["N"], qw, scale, 0, dev,
+                                   x=W.layer_input(pname, M, p["s"]), norm_weight=gf, eps=W.LAYER_NORM_EPS))
 
         def layer():
             for l in lins:
@@ -496,6 +577,9 @@ def main():
         return
     if args.quant_only:
         quant_only(dev, args.steps, args.warmup)
+        return
+    if args.fp8_only:
+        fp8_only(dev, args.steps, args.warmup)
         return
 
     linears = build_w8a8_sweep(dev)
@@ -607,11 +691,18 @@ def main():
     else:
         result["cpu_baseline"] = None
 
+    del linears, prefill
+    torch.cuda.empty_cache()
+    # the other two parts of the metric, each with its own roofline object inside the headline's `roofline`
+    fp8_rows = details_fp8(dev)
+    awq_rows = details_awq(dev, full=not args.no_details)
+    result["roofline"]["fp8"] = roofline_fp8(fp8_rows)
+    result["roofline"]["w4a16"] = roofline_w4a16(awq_rows)
+    result["pct_fp8_mfma_peak_prefill"] = round(100 * result["roofline"]["fp8"]["frac"], 2)
+    result["pct_hbm_peak_w4a16_decode"] = round(100 * result["roofline"]["w4a16"]["frac"], 2)
     if not args.no_details:
-        del linears, prefill
-        torch.cuda.empty_cache()
-        result["details"]["fp8"] = details_fp8(dev)
-        result["details"]["awq_w4a16"] = details_awq(dev)
+        result["details"]["fp8"] = fp8_rows
+        result["details"]["awq_w4a16"] = awq_rows
         result["details"]["layer_stack_w8a8"] = details_layer(dev)
         result["details"]["rmsnorm_quant_i8"] = details_norm_quant(dev)
 

@@ -139,6 +139,9 @@ def load_quantized_weights(model: nn.Module, path: str, device=None) -> tuple[li
                 with torch.no_grad():
                     dst.copy_(src.to(dst.dtype))
                 seen.add(key)
+    for m in model.modules():   # cached fp8 casts of weights that were just overwritten
+        if hasattr(m, "invalidate_cache"):
+            m.invalidate_cache()
     if device is not None:
         model.to(device)
     return sorted(k for k in own if k not in seen), unexpected

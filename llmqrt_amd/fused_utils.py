@@ -2,10 +2,12 @@
 
 Mirrors ``fuse_qkv`` / ``fuse_linears`` of the reference (utils/fused_utils.py:43-104), which fuses AWQ
 modules only and leaves SmoothQuant and FP8-dynamic qkv unfused (its comment at :49 calls that homework).
-With dynamic per-token activation scales the fusion is exact for those two as well: the scales depend only
-on the shared input, so the fused module's output is the concatenation of the separate outputs bit for bit.
-Modules whose activation scale is a stored per-module constant (SmoothQuant per-tensor, FP8 static) are
-returned unfused, as in the reference.
+With dynamic per-token activation scales and per-channel weight scales the fusion is exact for those two as
+well: the scales depend only on the shared input, so the fused module's output is the concatenation of the
+separate outputs bit for bit.  Modules whose activation scale is a stored per-module constant (SmoothQuant
+per-tensor, FP8 static) are returned unfused, as in the reference, and so are FP8-dynamic modules with
+per_tensor=True: they quantize the activations per tensor, run the tensor-wise kernel and return the module's
+dtype, none of which a per-channel fused module reproduces exactly.
 """
 from __future__ import annotations
 
@@ -48,13 +50,15 @@ def fuse_linears(linears):
         fused.bias = _cat_bias(linears)
         return fused
     if kind is FP8DynamicLinear:
+        if any(l.per_tensor for l in linears):
+            return list(linears)  # per-tensor activation scale + tensor-wise kernel: not reproduced by a fused module
+        if any(l.dtype != first.dtype or l.qdtype != first.qdtype for l in linears):
+            raise RuntimeError("FP8 modules with different dtypes cannot be fused")
         dev = first.weight.device
         fused = FP8DynamicLinear(first.in_features, n_out, first.bias is not None, dev=dev, dtype=first.dtype,
                                  qdtype=first.qdtype, per_tensor=False)
         fused.weight.data = torch.cat([l.weight.data for l in linears], dim=0).contiguous()
-        # a per-tensor scale becomes that value repeated for each of the module's channels
-        fused.weight_scale.data = torch.cat(
-            [l.weight_scale.data.reshape(-1, 1).expand(l.out_features, 1) for l in linears], dim=0).contiguous()
+        fused.weight_scale.data = torch.cat([l.weight_scale.data.reshape(-1, 1) for l in linears], dim=0).contiguous()
         if first.bias is not None:
             fused.bias.data = _cat_bias(linears)
         return fused

@@ -86,18 +86,23 @@ class WQLinear_GEMM(LinearBase):
         if init_only:
             return awq_linear
         assert scales is not None and zeros is not None
-        # scales, zeros: [N, K/G]; intw[k, n] = round((W[n, k] + z * s) / s)   (linear_awq.py:165-186)
+        # scales, zeros: [K/G, N], the orientation the reference indexes (scale_zeros[idx // group_size] is a
+        # row of N values; zeros are packed along dim 1): intw[k, n] = round((W[n, k] + z * s) / s)
+        # (linear_awq.py:165-186)
         G = awq_linear.group_size
-        s = scales.t().contiguous()                        # [K/G, N]
-        awq_linear.scales = s.clone().half()
+        want = (linear.in_features // G, linear.out_features)
+        if tuple(scales.shape) != want or tuple(zeros.shape) != want:
+            raise RuntimeError(f"from_linear: scales and zeros must be [in_features // group_size, out_features] = "
+                               f"{list(want)}, got {list(scales.shape)} and {list(zeros.shape)}")
+        awq_linear.scales = scales.clone().half()
         if linear.bias is not None:
             awq_linear.bias = linear.bias.clone().half()
-        sz = (zeros * scales).t().contiguous()             # [K/G, N]
+        sz = zeros * scales                                # [K/G, N]
         w_kn = linear.weight.data.t()                      # [K, N]
         intw = torch.round((w_kn + sz.repeat_interleave(G, dim=0)) /
                            awq_linear.scales.repeat_interleave(G, dim=0)).to(torch.int32)
         awq_linear.qweight = _pack_rows(intw, w_bit)
-        awq_linear.qzeros = _pack_rows(zeros.t().contiguous().to(torch.int32), w_bit)
+        awq_linear.qzeros = _pack_rows(zeros.to(torch.int32), w_bit)
         return awq_linear
 
     def forward(self, x):

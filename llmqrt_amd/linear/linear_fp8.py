@@ -37,12 +37,26 @@ class _FP8LinearBase(LinearBase):
         self._q_cache = None
 
     def _qweight_t(self):
-        """[K, N] column-major fp8 view of the weight, cast once per parameter version."""
+        """[K, N] column-major fp8 view of the weight.  The cast is made once and kept until the parameter is
+        replaced, moved, re-versioned (an in-place op on the Parameter) or a state dict is loaded; a write
+        through ``weight.data`` changes none of these and needs an explicit ``invalidate_cache()``."""
         w = self.weight
-        key = (w.data_ptr(), w._version, w.device)
+        key = (id(w), w.data_ptr(), w._version, w.device)
         if self._q_cache is None or self._q_cache[0] != key:
             self._q_cache = (key, w.detach().to(self.qdtype).contiguous())
         return self._q_cache[1].t()
+
+    def invalidate_cache(self):
+        """Drop the cached fp8 copy of the weight; the next forward casts again."""
+        self._q_cache = None
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self._q_cache = None   # loaders fill parameters through .data.copy_(), which bumps no version
+        return super()._load_from_state_dict(*args, **kwargs)
+
+    def _apply(self, fn, *args, **kwargs):
+        self._q_cache = None   # .to() / .cuda() / .half() replace or rewrite the parameter storage
+        return super()._apply(fn, *args, **kwargs)
 
 
 class FP8DynamicLinear(_FP8LinearBase):

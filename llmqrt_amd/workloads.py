@@ -85,6 +85,53 @@ def smoothquant_factors(x_absmax: torch.Tensor, w_absmax: torch.Tensor, alpha: f
     return (x_absmax.clamp(min=1e-5).pow(alpha) / w_absmax.clamp(min=1e-5).pow(1 - alpha)).clamp(min=1e-5)
 
 
+LAYER_M = (2048, 32)          # prefill tokens, decode batch
+LAYER_NORM_EPS = 1e-6
+# the two projections that read the output of an RMSNorm (input_layernorm -> qkv, post_attention_layernorm
+# -> gate_up); o and down read the attention / activation-function output, whose smoothing factors live in
+# the weights of the producer (v_proj, up_proj) and so arrive already divided
+LAYER_NORMED = ("qkv", "gate_up")
+
+
+def smoothquant_layer(alpha: float = 0.5, calib_tokens: int = 256, dtype=torch.bfloat16):
+    """One Qwen2-7B-shaped decoder layer's linears in SmoothQuant W8A8 form (all tensors on the CPU).
+
+    Per projection: dense fp32 weights W [N, K]; a seeded calibration batch gives max|X_j|; s from
+    smoothquant_factors; the int8 weights are the per-channel quantization of W * s; for the projections
+    behind an RMSNorm the norm weight g is stored both plain and folded (g / s, rounded to `dtype`), so that
+    norm_folded(x) = norm(x) / s feeds the quantizer directly.
+    -> {name: {K, N, w (fp32), s, qweight, w_scale, norm_weight, norm_weight_folded}}"""
+    layer = {}
+    for pi, (pname, (K, N)) in enumerate(QWEN2_7B_PROJ.items()):
+        w = dense_weights(N, K, seed_for(4, 100 + pi))
+        calib = activations(calib_tokens, K, seed_for(4, 200 + pi)).float()
+        g = gf = None
+        if pname in LAYER_NORMED:
+            g = (1.0 + 0.1 * torch.randn(K, generator=_gen(seed_for(4, 300 + pi)))).to(dtype)
+            inv = torch.rsqrt(calib.pow(2).mean(-1, keepdim=True) + LAYER_NORM_EPS)
+            calib = g.float() * (calib * inv)
+        s = smoothquant_factors(calib.abs().amax(0), w.abs().amax(0), alpha)
+        if g is not None:
+            gf = (g.float() / s).to(dtype)
+        ws = w * s.view(1, -1)
+        scale = ws.abs().amax(dim=1) / 127
+        qw = (ws / scale.view(-1, 1)).round_().clamp_(-128, 127).to(torch.int8)
+        layer[pname] = {"K": K, "N": N, "w": w, "s": s, "qweight": qw, "w_scale": scale,
+                        "norm_weight": g, "norm_weight_folded": gf}
+    return layer
+
+
+def layer_input(pname: str, M: int, s: torch.Tensor, dtype=torch.bfloat16) -> torch.Tensor:
+    """Input of projection `pname` of the layer stack for M tokens: the residual stream (in front of the
+    RMSNorm) for qkv / gate_up, the producer's output already divided by s for o / down."""
+    pi = list(QWEN2_7B_PROJ).index(pname)
+    K = QWEN2_7B_PROJ[pname][0]
+    x = activations(M, K, seed_for(4, 10 * pi + (0 if M > 64 else 1)), dtype=torch.float32)
+    if pname not in LAYER_NORMED:
+        x = x / s.view(1, -1)
+    return x.to(dtype)
+
+
 # ---- algorithmic work per linear (what the roofline figures are computed from) ---------------
 def gemm_ops(M, N, K) -> int:
     return 2 * M * N * K

@@ -98,14 +98,25 @@ def w8a8_epilogue_per_tensor(acc, bias, alpha: float, beta: float, out_dtype):
 
 @torch.no_grad()
 def w8a8_epilogue_per_token_per_channel(acc, a_scale, w_scale, bias, out_dtype):
-    """Per-token x per-channel dequant: utils/quantization_utils.py:89-97 gives
-    float(acc) * w_scale[n] * a_scale[m]; the op declared at csrc/smoothquant/sq_gemm.h:19-24
-    adds bias[n].  One rounding to out_dtype at the end, as in the reference's working
-    row-wise op (csrc/fp8/sm89_fp8_rowwise_fbgemm.cu:193-245)."""
+    """Epilogue of the per-token x per-channel op declared at csrc/smoothquant/sq_gemm.h:19-24 (body absent in
+    the reference).  Its semantics follow the reference's working per-token x per-channel op, the row-wise fp8
+    GEMM: ((float(acc) * a_scale[m]) * w_scale[n]) + bias[n], every node rounded to fp32, one rounding to
+    out_dtype at the end (the EVT tree at csrc/fp8/sm89_fp8_rowwise_fbgemm.cu:193-245).
+    dequantize_activation_w_per_channel_a_per_token below is the torch helper with the other multiplication
+    order; the two differ by at most one fp32 rounding before the final narrowing."""
     y = (acc.float() * a_scale.float().view(-1, 1)) * w_scale.float().view(1, -1)
     if bias is not None:
         y = y + bias.float().view(1, -1)
     return y.to(out_dtype)
+
+
+@torch.no_grad()
+def dequantize_activation_w_per_channel_a_per_token(q_act, w_scales, a_scales):
+    """utils/quantization_utils.py:89-97, line by line: (float(acc) * w_scale[n]) * a_scale[m] -> a_scales.dtype."""
+    dtype = a_scales.dtype
+    q_act = q_act.to(torch.float32)
+    q_act = q_act.mul(w_scales.reshape(1, -1)).mul(a_scales.reshape(-1, 1))
+    return q_act.to(dtype)
 
 
 @torch.no_grad()

@@ -108,22 +108,31 @@ def test_registry_and_module_interfaces():
 
 
 def test_awq_module_packer_matches_oracle():
+    """from_linear takes scales / zeros as [K/G, N], the orientation the reference indexes
+    (linear_awq.py:165-186, 203-219); N != K/G here so a transposed argument cannot pass unnoticed."""
     from llmqrt_amd.linear import WQLinear_GEMM
     from oracle import ref_math as R
     g = torch.Generator().manual_seed(0)
     lin = torch.nn.Linear(128, 64, bias=False)
     lin.weight.data = 0.02 * torch.randn(64, 128, generator=g)
     G = 64
-    wg = lin.weight.data.view(64, 2, G)
-    mx, mn = wg.amax(-1), wg.amin(-1)
-    scales = ((mx - mn) / 15).clamp(min=1e-5)                 # [N, K/G]
-    zeros = (-mn / scales).round().clamp(0, 15)               # [N, K/G]
+    wg = lin.weight.data.t().contiguous().view(2, G, 64)      # [K/G, G, N]
+    mx, mn = wg.amax(1), wg.amin(1)
+    scales = ((mx - mn) / 15).clamp(min=1e-5)                 # [K/G, N]
+    zeros = (-mn / scales).round().clamp(0, 15)               # [K/G, N]
     m = WQLinear_GEMM.from_linear(lin, 4, G, False, scales=scales, zeros=zeros)
+    assert m.scales.shape == (2, 64) and torch.equal(m.scales, scales.half())
     iw = R.awq_unpack(m.qweight)
     assert iw.min() >= 0 and iw.max() <= 15
-    assert torch.equal(R.awq_unpack(m.qzeros), zeros.t().int())
+    assert torch.equal(R.awq_unpack(m.qzeros), zeros.int())
+    # element by element against the reference's loop: intw[k, n] = round((W[n, k] + z s) / s)
+    for k, n in [(0, 0), (5, 63), (64, 1), (127, 40)]:
+        want = torch.round((lin.weight.data[n, k] + zeros[k // G, n] * scales[k // G, n]) / scales.half()[k // G, n])
+        assert iw[k, n] == int(want)
     deq = R.awq_dequantize(m.qweight, m.qzeros, m.scales, G)
     assert (deq.float() - lin.weight.data.t()).abs().max() <= 0.51 * scales.max()
+    with pytest.raises(RuntimeError, match="scales and zeros must be"):
+        WQLinear_GEMM.from_linear(lin, 4, G, False, scales=scales.t().contiguous(), zeros=zeros.t().contiguous())
 
 
 def test_workload_shapes_and_byte_counts():

@@ -378,3 +378,30 @@ def test_w8a8_full_prefill_size_properties(cuda):
     assert rel_err(fast[rows.to(cuda)], y_ref) <= REL_TOL
     doubled = w8a8_int8_linear_bbf16_obf16_per_channel(a, b, bias0, 2 * sxd, swd)
     assert torch.equal(doubled, 2 * fast)
+
+
+def test_fp8_full_prefill_size_properties(cuda):
+    """The largest FP8 launch of the benchmark (M = 4096, gate_up: N = 37888, K = 3584) on the benchmark's own
+    distribution (outlier-channel activations through the per-token fp8 quantizer, per-channel fp8 weights):
+    48 sampled token rows of the fp32 accumulators and of the outputs against the oracle, the fast epilogue equal
+    to the general one on all 155 M outputs, and exact scale linearity (doubling x_scale doubles every output)."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.sq_fp8_kernels import cutlass_f8f8bf16_rowwise_sm89
+    M, N, K = 4096, 37888, 3584
+    x = W.activations(M, K, W.seed_for(2, 22))
+    xq, xs = R.fp8_per_token_quantize(x)
+    wq, ws = W.fp8_weights(N, K, W.seed_for(2, 102))
+    a, b = xq.to(cuda), wq.to(cuda).t()
+    xsd, wsd = xs.to(cuda), ws.to(cuda).view(1, -1)
+    dump = torch.empty((M, N), dtype=torch.float32, device=cuda)
+    general = cutlass_f8f8bf16_rowwise_sm89(a, b, None, xsd, wsd, True, _acc_dump=dump)
+    fast = cutlass_f8f8bf16_rowwise_sm89(a, b, None, xsd, wsd, True)
+    assert torch.equal(fast.view(torch.int16), general.view(torch.int16))
+    rows = torch.arange(3, M, M // 48)
+    acc_ref = R.fp8_gemm_acc(xq[rows], wq)
+    assert rel_err(dump[rows.to(cuda)], acc_ref) <= FP8_ACC_TOL
+    y_ref = R.fp8_epilogue_rowwise(acc_ref, xs[rows], ws, None)
+    assert rel_err(fast[rows.to(cuda)], y_ref) <= REL_TOL
+    assert rel_err(fast[rows.to(cuda)], R.fp8_linear_naive(xq[rows], xs[rows], wq, ws, None)) <= REL_TOL
+    doubled = cutlass_f8f8bf16_rowwise_sm89(a, b, None, 2 * xsd, wsd, True)
+    assert torch.equal(doubled, 2 * fast)

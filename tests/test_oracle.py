@@ -167,6 +167,29 @@ def test_epilogue_invariants():
     assert torch.allclose(a, b, rtol=1e-5, atol=1e-3)
 
 
+def test_epilogue_multiplication_order():
+    """The reference's torch helper multiplies (acc * w_scale) * a_scale (utils/quantization_utils.py:89-97), the
+    op's epilogue (acc * a_scale) * w_scale (the row-wise fp8 op's tree).  Both round each fp32 product once:
+    they agree to 2 fp32 ulps, are identical for power-of-two scales, and after narrowing to bf16 differ in
+    at most a vanishing fraction of elements by one bf16 step."""
+    g = torch.Generator().manual_seed(4)
+    acc = torch.randint(-2000000, 2000000, (64, 96), generator=g).int()
+    sa, sw = torch.rand(64, generator=g) * 0.05 + 1e-3, torch.rand(96, generator=g) * 0.01 + 1e-4
+    a = R.w8a8_epilogue_per_token_per_channel(acc, sa, sw, None, torch.float32)
+    b = R.dequantize_activation_w_per_channel_a_per_token(acc, sw, sa.view(-1, 1))
+    assert b.dtype == torch.float32 and ((a - b).abs() <= 2.5e-7 * a.abs()).all()
+    p2a, p2w = 2.0 ** torch.randint(-8, 0, (64,), generator=g), 2.0 ** torch.randint(-10, -2, (96,), generator=g)
+    assert torch.equal(R.w8a8_epilogue_per_token_per_channel(acc, p2a, p2w, None, torch.float32),
+                       R.dequantize_activation_w_per_channel_a_per_token(acc, p2w, p2a.view(-1, 1)))
+    a16 = R.w8a8_epilogue_per_token_per_channel(acc, sa, sw, None, torch.bfloat16)
+    b16 = R.dequantize_activation_w_per_channel_a_per_token(acc, sw, sa.view(-1, 1).bfloat16().float()).bfloat16()
+    # (a_scales given in bf16 selects a bf16 result in the helper; compared on the same fp32 scale values)
+    a16b = R.w8a8_epilogue_per_token_per_channel(acc, sa.bfloat16().float(), sw, None, torch.bfloat16)
+    assert (a16b != b16).float().mean() < 1e-3
+    assert ((a16b.float() - b16.float()).abs() <= 2.0 ** -7 * b16.float().abs()).all()
+    assert a16.dtype == torch.bfloat16
+
+
 def test_reference_recipe_tolerance_sq():
     """unittest/test_sq_linear.py:8-34: the per-tensor op is within atol 0.1 of an fp16 Linear."""
     g = torch.Generator().manual_seed(0)
