@@ -485,10 +485,10 @@ def details_layer(dev):
             lins.append(W8A8Linear(f"{pname}_M{M}", M, p["K"], p["N"], qw, scale, 0, dev,
                                    x=W.layer_input(pname, M, p["s"]), norm_weight=gf, eps=W.LAYER_NORM_EPS))
 
-        def layer():
+        def run_layer():
             for l in lins:
                 l.launch(stream)
-        t = batch_time_us([layer], stream_obj, 10)
+        t = batch_time_us([run_layer], stream_obj, 10)
         ops = sum(l.ops for l in lins)
         per = {}
         for l in lins:
@@ -698,6 +698,10 @@ def main():
     awq_rows = details_awq(dev, full=not args.no_details)
     result["roofline"]["fp8"] = roofline_fp8(fp8_rows)
     result["roofline"]["w4a16"] = roofline_w4a16(awq_rows)
+    for part in ("fp8", "w4a16"):  # the same figures as flat scalars, for readers that keep only scalar fields
+        for key in ("achieved", "frac", "avg_launch_us", "traffic"):
+            result["roofline"][f"{part}_{key}"] = result["roofline"][part][key]
+        result["roofline"][f"{part}_unit"] = result["roofline"][part]["unit"]
     result["pct_fp8_mfma_peak_prefill"] = round(100 * result["roofline"]["fp8"]["frac"], 2)
     result["pct_hbm_peak_w4a16_decode"] = round(100 * result["roofline"]["w4a16"]["frac"], 2)
     if not args.no_details:

@@ -47,8 +47,10 @@ def test_fuse_sq_per_channel(cuda, M):
     assert _rel(got, ref) <= OUT_TOL
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_fuse_fp8_dynamic_per_channel(cuda, dtype):
+def test_fuse_fp8_dynamic_per_channel(cuda):
+    # bf16 only: the row-wise op returns bf16 and takes a bf16 / fp32 bias, as the reference's does
+    # (csrc/fp8/sm89_fp8_rowwise_fbgemm.cu:286-287,560-566)
+    dtype = torch.bfloat16
     from llmqrt_amd.fused_utils import fuse_linears
     from llmqrt_amd.linear import FP8DynamicLinear
     mods = [FP8DynamicLinear.from_linear(_dense(n, K, 20 + i).to(cuda), init_only=False, dtype=dtype,

@@ -11,10 +11,11 @@ from oracle import ref_math as R
 pytestmark = pytest.mark.gpu
 REL_TOL = 1e-2
 # fp32 accumulators of the fp8 MFMA against an fp64 sum of the same exact products, relative to the
-# largest accumulator.  One v_mfma_f32_32x32x64_f8f6f4 adds its 64 products in a fixed-point window
-# below the largest of them (measured: errors up to ~5e-5 of the largest accumulator at K = 3584), the
-# same class of arithmetic as the reference's use_fast_accum=True tensor-core path; between
-# instructions the accumulation is plain fp32.
+# largest accumulator.  v_mfma_f32_32x32x64_f8f6f4 sums each run of 8 consecutive k in fixed point below
+# the largest product of the run: a product more than 13 binary orders below it is dropped
+# (test_fp8_mfma_accumulation_window pins this with known answers).  That bounds one instruction's error
+# by 7 * 2^-14 = 4.3e-4 of its largest product; on the benchmark's data the accumulators end up within
+# ~5e-5 of the exact sum.  The reference's use_fast_accum=True tensor-core path is the same class of arithmetic.
 FP8_ACC_TOL = 2e-4
 
 
@@ -209,6 +210,36 @@ def test_fp8_reference_recipes(cuda):
     out16 = cutlass_f8f8bf16_tensorwise_sm89(a.to(cuda), b.to(cuda).t(), None, 0.6, 1, "float16")
     assert out16.dtype == torch.float16
     assert rel_err(out16, (0.6 * (a.float() @ b.float().t())).half()) <= REL_TOL
+
+
+def test_fp8_mfma_accumulation_window(cuda):
+    """Known answers for how the fp8 matrix instruction adds its products: one large product (k = 0) and 63
+    equal small ones.  Small products down to 2^-13 of the large one are all kept (the sum is exact); at 2^-14
+    exactly the 7 that share the large product's run of 8 consecutive k are dropped, the other 56 are kept; the
+    sum of the small ones alone is exact at any magnitude.  This is what FP8_ACC_TOL allows for."""
+    from llmqrt_amd.sq_fp8_kernels import cutlass_f8f8bf16_rowwise_sm89
+    M = N = 32
+    ones_m, ones_n = torch.ones(M, 1, device=cuda), torch.ones(1, N, device=cuda)
+
+    def acc_of(big_a, big_b, small_a, small_b, K=64):
+        a, b = torch.zeros(M, K), torch.zeros(N, K)
+        a[:, 0], b[:, 0] = big_a, big_b
+        a[:, 1:64], b[:, 1:64] = small_a, small_b
+        dump = torch.empty((M, N), dtype=torch.float32, device=cuda)
+        cutlass_f8f8bf16_rowwise_sm89(a.to(torch.float8_e4m3fn).to(cuda), b.to(torch.float8_e4m3fn).to(cuda).t(), None,
+                                      ones_m, ones_n, True, _acc_dump=dump)
+        assert (dump == dump[0, 0]).all()
+        return dump[0, 0].item()
+    big = 2.0 ** 8                                                  # 16 * 16
+    assert acc_of(16, 16, 2.0 ** -2, 2.0 ** -3) == big + 63 * 2.0 ** -5      # 2^-13 of the large product: exact
+    assert acc_of(16, 16, 2.0 ** -3, 2.0 ** -3) == big + 56 * 2.0 ** -6      # 2^-14: the 7 run-mates are dropped
+    assert acc_of(0, 0, 2.0 ** -3, 2.0 ** -3) == 63 * 2.0 ** -6              # no large product: exact
+    assert acc_of(16, 16, 2.0 ** -3, 2.0 ** -3, K=128) == big + 56 * 2.0 ** -6   # zero tail tile changes nothing
+    # the bound used by the tolerance: never worse than 7 dropped run-mates
+    for t in range(4, 12):
+        got = acc_of(16, 16, 2.0 ** -(t // 2), 2.0 ** -(t - t // 2))
+        exact = big + 63 * 2.0 ** -t
+        assert exact - 7 * 2.0 ** -t <= got <= exact
 
 
 def test_fp8_e5m2_activations(cuda):
