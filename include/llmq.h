@@ -30,7 +30,8 @@ typedef enum {
     LLMQ_ERR_SHAPE = -3,     /* negative size, stride smaller than the row, unsupported alignment */
     LLMQ_ERR_WORKSPACE = -4, /* workspace missing or too small */
     LLMQ_ERR_LAUNCH = -5,    /* the HIP runtime refused the launch (hipGetLastError) */
-    LLMQ_ERR_ALIGN = -6      /* a pointer is not 16-byte aligned */
+    LLMQ_ERR_ALIGN = -6,     /* a pointer is not 16-byte aligned */
+    LLMQ_ERR_SCRATCH = -7    /* the problem needs more scratch than the library's static array holds */
 } llmq_status;
 
 typedef enum { LLMQ_BF16 = 0, LLMQ_F16 = 1, LLMQ_F32 = 2 } llmq_dtype;
@@ -148,6 +149,23 @@ int llmq_gemm_fp8(const uint8_t* A, int a_format, int64_t lda, const uint8_t* B,
                   llmq_stream_t stream);
 
 size_t llmq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/* llmq_gemm_w8a8 for callers that cannot allocate or pass a workspace: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments and
+ * results as llmq_gemm_w8a8 without acc_dump / workspace: the split-K partial sums go to a static device array
+ * of llmq_gemm_static_scratch_bytes() (32 MiB) that every GPU holds from library load to process exit.  The
+ * call allocates nothing (no hipMalloc / hipFree), looks the array's device address up once per device (on the
+ * first call there: make that call outside a graph capture) and returns LLMQ_ERR_SCRATCH when
+ * llmq_gemm_workspace_bytes(M, N, K) exceeds the array.  All calls on one GPU share the array: two calls that
+ * overlap in time (different streams) race; calls on one stream are ordered and safe.  Nothing in the array has
+ * to start at zero: every partial sum is written before it is read. */
+int llmq_gemm_w8a8_static(const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb,
+                          const float* a_scale, const float* w_scale,
+                          float alpha, const float* alpha_dev,
+                          const void* bias, int bias_dtype, float beta,
+                          void* out, int out_dtype, int64_t ldo,
+                          int64_t M, int64_t N, int64_t K, llmq_stream_t stream);
+size_t llmq_gemm_static_scratch_bytes(void);
 
 /* Tuning / test hook with no counterpart in the reference: force tile configuration `cfg`
  * (0 .. llmq_gemm_num_configs()-1) and K split `splits` for every later GEMM call of this

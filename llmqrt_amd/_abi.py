@@ -38,6 +38,9 @@ SIGNATURES = {
     "llmq_gemm_fp8": (_int, [_vp, _int, _i64, _vp, _i64, _vp, _vp, _f32, _vp, _vp, _int, _f32, _vp, _int, _i64,
                              _i64, _i64, _i64, _vp, _vp, _sz, _vp]),
     "llmq_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "llmq_gemm_w8a8_static": (_int, [_vp, _i64, _vp, _i64, _vp, _vp, _f32, _vp, _vp, _int, _f32, _vp, _int, _i64,
+                                     _i64, _i64, _i64, _vp]),
+    "llmq_gemm_static_scratch_bytes": (_sz, []),
     "llmq_gemm_force_plan": (_int, [_int, _int]),
     "llmq_gemm_num_configs": (_int, []),
     "llmq_awq_gemm": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),

@@ -12,6 +12,7 @@ extern "C" const char* llmq_status_string(int status) {
         case LLMQ_ERR_WORKSPACE: return "workspace missing or too small";
         case LLMQ_ERR_LAUNCH: return "HIP launch failed";
         case LLMQ_ERR_ALIGN: return "pointer is not sufficiently aligned";
+        case LLMQ_ERR_SCRATCH: return "problem needs more scratch than the library's static array holds";
         default: return "unknown status";
     }
 }

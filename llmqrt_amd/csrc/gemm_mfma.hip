@@ -732,10 +732,48 @@ int gemm_entry(bool fp8, int a_format, const uint8_t* A, int64_t lda, const uint
     return launch_gemm<true, 1>(A, lda, B, ldb, (int)M, (int)N, (int)K, p, ep, out, ldo, acc_dump, ws, st);
 }
 
+// ---- scratch owned by the library, for the entry point that takes no workspace ---------------------
+// One copy of this array exists on every GPU the library is loaded on, for the life of the process.
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+// `scratch` is a host-side stand-in for the symbol, not a device address: the address of each GPU's copy
+// is looked up once per device and only that pointer is ever handed to a kernel.
+void* g_scratch_ptr[64] = {};
+
+int static_scratch(void** out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LLMQ_ERR_LAUNCH;
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return LLMQ_ERR_LAUNCH;
+        g_scratch_ptr[dev] = p;  // benign if two threads race here: both store the same address
+    }
+    *out = g_scratch_ptr[dev];
+    return LLMQ_OK;
+}
+
 }  // namespace
 }  // namespace llmq
 
 using namespace llmq;
+
+extern "C" size_t llmq_gemm_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int llmq_gemm_w8a8_static(const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb, const float* a_scale,
+                                     const float* w_scale, float alpha, const float* alpha_dev, const void* bias,
+                                     int bias_dtype, float beta, void* out, int out_dtype, int64_t ldo, int64_t M,
+                                     int64_t N, int64_t K, llmq_stream_t stream) {
+    if (M > 0 && N > 0 && K > 0) {
+        const Plan p = make_plan(M, N, K);
+        if (p.splits > 1 && (size_t)p.splits * M * N * 4 > kStaticScratchBytes) return LLMQ_ERR_SCRATCH;
+    }
+    void* ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc != LLMQ_OK) return rc;
+    return gemm_entry(false, 0, (const uint8_t*)A, lda, (const uint8_t*)B, ldb, a_scale, w_scale, alpha, alpha_dev,
+                      bias, bias_dtype, beta, out, out_dtype, ldo, M, N, K, nullptr, ws, kStaticScratchBytes,
+                      (hipStream_t)stream);
+}
 
 extern "C" int llmq_gemm_force_plan(int cfg, int splits) {
     if (cfg >= kNumShapes || splits < 1 || splits > 64) return LLMQ_ERR_SHAPE;
