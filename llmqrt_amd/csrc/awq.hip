@@ -31,6 +31,15 @@ int launch_awq_tile(const AwqTilePlan& p, const uint16_t* x, int64_t ldx, const 
                     const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K, int G,
                     hipStream_t st);
 
+// Decode kernel for up to 16 tokens (awq_decode.hip).
+struct AwqDecodePlan { int cs, pd, splits, groups_per_block; };
+bool awq_decode_supported(int64_t M, int64_t N, int64_t K, int64_t group);
+AwqDecodePlan make_awq_decode_plan(int64_t M, int64_t N, int64_t K, int force_cs, int force_pd, int force_splits);
+size_t awq_decode_workspace_bytes(const AwqDecodePlan& p, int64_t M, int64_t N);
+int launch_awq_decode(const AwqDecodePlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
+                      const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K,
+                      hipStream_t st);
+
 namespace {
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
@@ -691,6 +700,18 @@ DecodePlan make_decode_plan(int64_t M, int64_t N, int64_t K) {
 // The streaming kernel handles up to 64 tokens per weight pass as up to 4 slabs of 16.
 inline bool decode_path(int64_t M, int64_t group) { return M <= 64 && group == 128; }
 
+// The LDS-staged decode kernel (one launch, in-kernel K-split reduction) serves the first few tokens, where it is
+// ahead of the register-streaming kernel; llmq_awq_force_plan 8..11 picks its tile width and prefetch depth for any
+// M <= 16, 1 / 2 / 5 / 6 keep the register-streaming kernel.  Measured crossover: 4 tokens (2 for a long K, where the
+// partial sums of the K split grow with the token count).
+inline bool decode16_path(int64_t M, int64_t N, int64_t K, int64_t group) {
+    return ((g_force_v == 0 && M <= (K >= 8192 ? 2 : 4)) || (g_force_v >= 8 && g_force_v <= 11)) && awq_decode_supported(M, N, K, group);
+}
+inline AwqDecodePlan decode16_plan(int64_t M, int64_t N, int64_t K) {
+    const int cs = g_force_v >= 8 ? ((g_force_v & 1) ? 4 : 2) : 0, pd = g_force_v >= 8 ? (g_force_v >= 10 ? 2 : 1) : 0;
+    return make_awq_decode_plan(M, N, K, cs, pd, g_force_splits);
+}
+
 // More than 64 tokens go to the tile kernel (weights dequantized once per token tile on their way into LDS);
 // llmq_awq_force_plan(3 | 4, ...) forces its 64x128 | 256x256 tile for any M, (1 | 2, ...) keeps the slabs.
 inline bool tile_path(int64_t M) { return g_force_v == 3 || g_force_v == 4 || g_force_v == 7 || (g_force_v == 0 && M > 64); }
@@ -713,7 +734,7 @@ void launch_awq(const AwqPlan& p, const uint16_t* x, int64_t ldx, const uint32_t
 using namespace llmq;
 
 extern "C" int llmq_awq_force_plan(int v, int splits, int k_waves) {
-    if (v < 0 || v > 7 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
+    if (v < 0 || v > 11 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 2 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
     g_force_v = v;
     g_force_splits = splits;
     g_force_kw = k_waves;
@@ -726,6 +747,10 @@ extern "C" size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
     if (tile_path(M)) {
         const AwqTilePlan t = tile_plan(M, N, K);
         if (t.splits > 1) total = (size_t)t.splits * M * N * sizeof(float);
+    }
+    if (M <= 16 && awq_decode_supported(M, N, K, 128)) {
+        const size_t need = awq_decode_workspace_bytes(decode16_plan(M, N, K), M, N);
+        if (need > total) total = need;
     }
     for (int64_t m0 = 0; m0 < M; m0 += 64) {
         const int64_t mm = M - m0 < 64 ? M - m0 : 64;
@@ -773,6 +798,11 @@ extern "C" int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight,
             if (launch_status() != LLMQ_OK) return LLMQ_ERR_LAUNCH;
         }
         return LLMQ_OK;
+    }
+    if (decode16_path(M, N, K, group)) {
+        const AwqDecodePlan d = decode16_plan(M, N, K);
+        if (d.splits > 1 && (!ws || workspace_bytes < awq_decode_workspace_bytes(d, M, N))) return LLMQ_ERR_WORKSPACE;
+        return launch_awq_decode(d, (const uint16_t*)x, ldx, qw, sc, qz, bs, (uint16_t*)out, ws, (int)M, Ni, Ki, st);
     }
     // tokens are processed in slabs of at most 64 rows (4 MFMA token tiles per weight pass)
     for (int64_t m0 = 0; m0 < M; m0 += 64) {

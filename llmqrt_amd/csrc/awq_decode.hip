@@ -1,0 +1,417 @@
+// AWQ W4A16 decode kernel: up to 16 tokens, group size 128, N a multiple of 32.
+//
+// The op is a stream of half a byte per weight out of HBM, so the kernel is laid out around the memory
+// system first.  Measured on MI355X with a pure-load kernel over the [K, N/8] int32 weight matrix: a
+// wavefront load that covers 64-byte row segments streams at 2.5-3.2 TB/s, one that covers whole 128-byte
+// lines with 16 bytes per lane at 5.3-5.8 TB/s, provided a few thousand wavefronts each keep about four such
+// loads in flight.  Hence:
+//   * A block of CS wavefronts owns a column tile of 16*CS packed words (128 or 256 bytes per row) and a run
+//     of whole quantization groups along K.  The tile moves in stages of 64 rows: every thread fetches four
+//     16-byte pieces (a wavefront instruction covers 4-8 rows x 128-256 contiguous bytes), PD stages ahead of
+//     the one being computed, and drops them into a double-buffered LDS tile.
+//   * Compute reads LDS in the layout the matrix core wants: wavefront w owns word columns 16w .. 16w+15, a
+//     lane the 8 consecutive k-rows of one word column, i.e. an 8x8 block of nibbles = the operand of 8
+//     v_mfma_f32_16x16x32_f16 (tokens x 16 channels x 32 k), one per logical column of the word.
+//   * Nibbles are not converted: v_perm_b32 puts the same byte of two k-adjacent words into bytes 0 / 2 of a
+//     register; masked with 0x000F000F / 0x00F000F0 the nibbles read as fp16 subnormals q * 2^-24 /
+//     16 q * 2^-24, which the matrix core multiplies exactly.  Scale and zero point are applied once per
+//     group and output: y += s * 2^24 * acc - s * z * sum_k(x), with sum_k(x) from one MFMA against ones.
+//     (0.75 VALU operations per weight plus 64 per group and wavefront.)
+//   * A K split across blocks writes fp32 partial sums [split][M][N] to the caller's workspace; the block that
+//     arrives last at a column tile adds them in split order and writes the output: one launch, results
+//     independent of scheduling.  Arrivals are counted in a ring of self-resetting tickets that the library owns
+//     (a zero-initialised static device array; every call takes fresh slots, so concurrent calls do not share any).
+#include <atomic>
+#include <type_traits>
+
+#include "llmq_common.h"
+
+namespace llmq {
+
+struct AwqDecodePlan { int cs, pd, splits, groups_per_block; };
+
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));  // a first-class 16-byte value (HIP's uint4 is a struct: copies of it become memcpy)
+
+constexpr int kGroup = 128;      // quantization group = 2 stages of 64 rows = 4 MFMA chunks of 32 rows
+constexpr int kStageRows = 64;
+
+__host__ __device__ constexpr int rev_nibble_d(int j) { return ((j & 1) << 2) | (j >> 1); }  // {0,4,1,5,2,6,3,7}
+
+// Cross-block end of a K split, shared by the decode kernels.  On entry `ptile` (LDS, [M][TILE_CH] fp32) holds this
+// block's partial sums for column tile `tile` and every thread of the block has passed a barrier after writing it.
+// Every block publishes its tile to partials[ks][M][N]; the block that arrives last at the tile adds the splits in
+// split order (so the result does not depend on which block that is), adds the bias and writes the output.
+// Cross-block visibility without cache-wide fences (a device-scope release fence writes back the whole L2 of the
+// XCD: measured at ~100 us per launch): the partial sums are stored and loaded with the device-coherent cache
+// policy (sc1: written through / not served from another XCD's stale copy), every wavefront waits until its stores
+// have completed before the block takes its ticket, and the ticket is a device-scope atomic.  The coherent stores
+// are whole 16-byte pieces of 128-byte lines (4-byte write-through pieces were measured at +11 us per launch).
+// Tickets of neighbouring tiles are 256 bytes apart so that their atomics land in different memory channels
+// (adjacent words were measured 1-3 us slower per launch).
+constexpr int kTicketStride = 64;  // in 4-byte words
+constexpr int kTicketRing = 1 << 18;  // words in the ring of tickets
+template <int TILE_CH, int NT>
+__device__ __forceinline__ void finish_split_tile(const float* ptile, int M, int N, int tile, int ks, int splits,
+                                                  float* partials, unsigned int* tickets, const uint16_t* bias,
+                                                  uint16_t* out) {
+    const int tid = threadIdx.x;
+    const int tile_n0 = tile * TILE_CH;                  // first channel of the tile
+    const int tile_q = min(TILE_CH, N - tile_n0) >> 2;   // its width in units of 4 channels (N % 32 == 0)
+    auto store4 = [&](v4f acc, int m, int nn) __attribute__((always_inline)) {
+        float lo0 = acc[0], hi0 = acc[1], lo1 = acc[2], hi1 = acc[3];
+        if (bias) {
+            lo0 = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(lo0)) + Lo<LLMQ_F16>::to_f32(bias[nn]);
+            hi0 = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(hi0)) + Lo<LLMQ_F16>::to_f32(bias[nn + 1]);
+            lo1 = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(lo1)) + Lo<LLMQ_F16>::to_f32(bias[nn + 2]);
+            hi1 = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(hi1)) + Lo<LLMQ_F16>::to_f32(bias[nn + 3]);
+        }
+        *reinterpret_cast<uint2*>(out + (int64_t)m * N + nn) =
+            make_uint2((uint32_t)Lo<LLMQ_F16>::from_f32(lo0) | ((uint32_t)Lo<LLMQ_F16>::from_f32(hi0) << 16),
+                       (uint32_t)Lo<LLMQ_F16>::from_f32(lo1) | ((uint32_t)Lo<LLMQ_F16>::from_f32(hi1) << 16));
+    };
+    if (splits == 1) {
+        for (int idx = tid; idx < M * tile_q; idx += NT) {
+            const int m = idx / tile_q, c4 = idx - m * tile_q;
+            store4(*reinterpret_cast<const v4f*>(ptile + m * TILE_CH + 4 * c4), m, tile_n0 + 4 * c4);
+        }
+        return;
+    }
+    for (int idx = tid; idx < M * tile_q; idx += NT) {
+        const int m = idx / tile_q, c4 = idx - m * tile_q;
+        const v4f v = *reinterpret_cast<const v4f*>(ptile + m * TILE_CH + 4 * c4);
+        float* dst = partials + ((int64_t)ks * M + m) * N + tile_n0 + 4 * c4;
+        asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's coherent stores have completed
+    __shared__ int s_last;
+    __syncthreads();
+    if (tid == 0) {
+        // Arrival ticket of this column tile: counts 0 .. splits-1 and wraps back to 0 with the last arrival, so the
+        // slot is clean again for whichever call gets it next.  One atomic per block, no retry loop (a
+        // compare-and-swap loop on a shared word was measured at ~1.5 us per arrival, serialized).
+        s_last = atomicInc(tickets + kTicketStride * tile, (unsigned)(splits - 1)) == (unsigned)(splits - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    for (int idx = tid; idx < M * tile_q; idx += NT) {
+        const int m = idx / tile_q, nn = tile_n0 + 4 * (idx - m * tile_q);
+        const float* src = partials + (int64_t)m * N + nn;
+        const int64_t sstride = (int64_t)M * N;
+        v4f acc = {0.f, 0.f, 0.f, 0.f};
+        for (int sp = 0; sp < splits; sp += 8) {  // eight coherent loads in flight, added in split order
+            v4f t0, t1, t2, t3, t4, t5, t6, t7;
+            auto ld = [&](int i, v4f& t) __attribute__((always_inline)) {
+                const float* p = src + (int64_t)min(sp + i, splits - 1) * sstride;
+                asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(t) : "v"(p) : "memory");
+            };
+            ld(0, t0), ld(1, t1), ld(2, t2), ld(3, t3), ld(4, t4), ld(5, t5), ld(6, t6), ld(7, t7);
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(t0), "+v"(t1), "+v"(t2), "+v"(t3), "+v"(t4), "+v"(t5), "+v"(t6), "+v"(t7)::"memory");
+            const int left = splits - sp;
+            acc += t0;
+            if (left > 1) acc += t1;
+            if (left > 2) acc += t2;
+            if (left > 3) acc += t3;
+            if (left > 4) acc += t4;
+            if (left > 5) acc += t5;
+            if (left > 6) acc += t6;
+            if (left > 7) acc += t7;
+        }
+        store4(acc, m, nn);
+    }
+}
+
+template <int CS, int PD, int RM>  // RM: token rows per lane that can be live (min(M, 4))
+__global__ __launch_bounds__(CS * kWave, 3) void awq_decode_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, const uint32_t* __restrict__ qw,
+    const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qz, const uint16_t* __restrict__ bias,
+    uint16_t* __restrict__ out, float* partials, unsigned int* tickets, int M, int N, int K, int gpb, int tiles_n) {
+    constexpr int NT = CS * kWave, SEGW = 16 * CS, SEGQ = SEGW / 4;  // words / 16-byte pieces per tile row
+    constexpr int RPL = NT / SEGQ;                                   // rows one block-wide load covers (16)
+    constexpr int LOADS = kStageRows / RPL;                          // 16-byte loads per thread and stage (4)
+    constexpr int STRIDE = SEGW + 4;  // LDS row stride in words: keeps 16-byte alignment, spreads rows 8 apart over banks
+    static_assert(RPL == 16 && LOADS == 4, "a stage is four block-wide loads");
+    constexpr int XSTRIDE = 36;       // LDS row stride of the activation tile in words (64 k = 32 words + 4)
+    __shared__ __attribute__((aligned(16))) uint32_t lds[2][kStageRows * STRIDE];
+    __shared__ __attribute__((aligned(16))) uint32_t ldx_s[2][16 * XSTRIDE];  // 16 tokens x 64 k of fp16 per stage
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int li = lane & 15, kb = lane >> 4;
+    const int Nw = N >> 3, Nq = Nw >> 2;
+    const int tile = blockIdx.x % tiles_n, ks = blockIdx.x / tiles_n;
+    const int ngroups = K / kGroup;
+    const int g_begin = ks * gpb, g_end = min(ngroups, g_begin + gpb);
+    const int nst = 2 * (g_end - g_begin);
+
+    // ---- global -> register mapping of the cooperative tile load
+    const int ld_row = tid / SEGQ, ld_seg = tid % SEGQ;
+    const int colq = min(tile * SEGQ + ld_seg, Nq - 1);  // a tile past the ragged edge re-reads the last piece (unused)
+    const u4* wbase = reinterpret_cast<const u4*>(qw) + (int64_t)(g_begin * kGroup + ld_row) * Nq + colq;
+    const int st_slot = ld_row * STRIDE + 4 * ld_seg;
+
+    // ---- compute mapping
+    const int cw = tile * SEGW + 16 * wave + li;  // word column of this lane
+    const bool col_ok = cw < Nw;
+    const int cwc = col_ok ? cw : 0;
+    // activations: the first 128 threads fetch one 16-byte piece each of the stage's 16 tokens x 64 k
+    const bool x_loader = tid < 128;              // wavefront-uniform
+    const int x_tok = (tid >> 3) & 15, x_piece = tid & 7;
+    const bool x_ok = x_tok < M;
+    const uint8_t* xbase = reinterpret_cast<const uint8_t*>(x) +
+                           ((int64_t)min(x_tok, M - 1) * ldx + (int64_t)g_begin * kGroup + 8 * x_piece) * 2;
+    const int x_slot = x_tok * XSTRIDE + 4 * x_piece;
+
+    struct Stage { u4 w0, w1, w2, w3, x0; };  // one stage in flight: 4 weight pieces, 1 activation piece
+    Stage sa, sb;
+    uint32_t z_next;
+    u4 s_next;
+    // every load is unconditional: indices past the block's K range re-read its last stage / group
+    auto load_stage = [&](int s, Stage& d) __attribute__((always_inline)) {
+        s = min(s, nst - 1);
+        const u4* p = wbase + (int64_t)s * kStageRows * Nq;
+        d.w0 = p[0];
+        d.w1 = p[(int64_t)RPL * Nq];
+        d.w2 = p[(int64_t)2 * RPL * Nq];
+        d.w3 = p[(int64_t)3 * RPL * Nq];
+        if (x_loader) d.x0 = *reinterpret_cast<const u4*>(xbase + s * (kStageRows * 2));
+    };
+    auto load_group = [&](int g) __attribute__((always_inline)) {
+        g = min(g, g_end - 1);
+        z_next = qz[(int64_t)g * Nw + cwc];
+        s_next = *reinterpret_cast<const u4*>(scales + (int64_t)g * N + 8 * cwc);
+    };
+    auto lds_barrier = []() __attribute__((always_inline)) {  // orders LDS traffic only: the prefetched global loads stay in flight across it
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    };
+
+    v4f y[8], accg[8], xs = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 8; j++) y[j] = accg[j] = v4f{0.f, 0.f, 0.f, 0.f};
+    const h8 ones = {(_Float16)1.f, (_Float16)1.f, (_Float16)1.f, (_Float16)1.f,
+                     (_Float16)1.f, (_Float16)1.f, (_Float16)1.f, (_Float16)1.f};
+
+    load_group(g_begin);
+    load_stage(0, sa);
+    if constexpr (PD == 2) load_stage(1, sb);
+
+    uint32_t z_cur = 0;
+    u4 s_cur = {0u, 0u, 0u, 0u};
+
+    auto stage_body = [&](int st, Stage& cur) __attribute__((always_inline)) {  // cur: the register set that holds stage st
+        const int buf = st & 1;
+        uint32_t* tile_lds = lds[buf];
+        *reinterpret_cast<u4*>(tile_lds + st_slot) = cur.w0;
+        *reinterpret_cast<u4*>(tile_lds + st_slot + RPL * STRIDE) = cur.w1;
+        *reinterpret_cast<u4*>(tile_lds + st_slot + 2 * RPL * STRIDE) = cur.w2;
+        *reinterpret_cast<u4*>(tile_lds + st_slot + 3 * RPL * STRIDE) = cur.w3;
+        if (x_loader) *reinterpret_cast<u4*>(ldx_s[buf] + x_slot) = x_ok ? cur.x0 : u4{0u, 0u, 0u, 0u};  // rows past M read as 0
+        if ((st & 1) == 0) {
+            z_cur = z_next;
+            s_cur = s_next;
+            load_group(g_begin + (st >> 1) + 1);
+        }
+        load_stage(st + PD, cur);
+        lds_barrier();
+#pragma unroll
+        for (int c2 = 0; c2 < 2; c2++) {
+            const uint32_t* lp = tile_lds + (32 * c2 + 8 * kb) * STRIDE + 16 * wave + li;
+            uint32_t w[8];
+#pragma unroll
+            for (int r = 0; r < 8; r++) w[r] = lp[r * STRIDE];
+            // activation operand: token li, k = 32 c2 + 8 kb .. + 7
+            const h8 xb = __builtin_bit_cast(h8, *reinterpret_cast<const u4*>(ldx_s[buf] + li * XSTRIDE + 4 * (4 * c2 + kb)));
+            xs = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb, ones, xs, 0, 0, 0);
+#pragma unroll
+            for (int bsel = 0; bsel < 4; bsel++) {  // byte of the word: nibbles 2*bsel (low) and 2*bsel+1 (high)
+                const uint32_t sel = (uint32_t)bsel | 0x0c00u | ((uint32_t)(4 + bsel) << 16) | 0x0c000000u;
+                constexpr int kColOfNibble[8] = {0, 2, 4, 6, 1, 3, 5, 7};
+                const int jl = kColOfNibble[2 * bsel], jh = kColOfNibble[2 * bsel + 1];
+                uint32_t lo[4], hi[4];
+#pragma unroll
+                for (int pr = 0; pr < 4; pr++) {
+                    const uint32_t uu = __builtin_amdgcn_perm(w[2 * pr + 1], w[2 * pr], sel);  // byte0 <- row 2pr, byte2 <- row 2pr+1
+                    lo[pr] = uu & 0x000F000Fu;  // q_lo * 2^-24 as fp16 subnormals
+                    hi[pr] = uu;                // the whole byte: (16 q_hi + q_lo) * 2^-24, still subnormal and exact
+                }
+                const h8 bl = __builtin_bit_cast(h8, v4i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3]});
+                const h8 bh = __builtin_bit_cast(h8, v4i{(int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]});
+                accg[jl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb, bl, accg[jl], 0, 0, 0);
+                accg[jh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb, bh, accg[jh], 0, 0, 0);
+            }
+        }
+        if (st & 1) {
+            // Finished group.  Per byte of the word the accumulators hold L = sum x q_lo 2^-24 (low-nibble column jl)
+            // and U = sum x (16 q_hi + q_lo) 2^-24 (high-nibble column jh), so
+            //   y_jl += s_jl 2^24 L - s_jl z_jl sum(x),   y_jh += s_jh 2^20 (U - L) - s_jh z_jh sum(x);
+            // the group accumulators restart at 0.  Rows past RM belong to tokens past M: their operand rows are zero.
+            const uint32_t sw[4] = {s_cur[0], s_cur[1], s_cur[2], s_cur[3]};
+            auto scale_of = [&](int j) __attribute__((always_inline)) {
+                return Lo<LLMQ_F16>::to_f32((uint16_t)((j & 1) ? (sw[j >> 1] >> 16) : (sw[j >> 1] & 0xffffu)));
+            };
+#pragma unroll
+            for (int bsel = 0; bsel < 4; bsel++) {
+                constexpr int kColOfNibble[8] = {0, 2, 4, 6, 1, 3, 5, 7};
+                const int jl = kColOfNibble[2 * bsel], jh = kColOfNibble[2 * bsel + 1];
+                const float sl = scale_of(jl), sh = scale_of(jh);
+                const float zl = (float)((z_cur >> (8 * bsel)) & 0xFu), zh = (float)((z_cur >> (8 * bsel + 4)) & 0xFu);
+                const float sl24 = sl * 16777216.0f, sh20 = sh * 1048576.0f, nslz = -sl * zl, nshz = -sh * zh;
+#pragma unroll
+                for (int r = 0; r < RM; r++) {
+                    const float L = accg[jl][r], U = accg[jh][r];
+                    y[jl][r] = fmaf(sl24, L, fmaf(nslz, xs[r], y[jl][r]));
+                    y[jh][r] = fmaf(sh20, U, fmaf(-sh20, L, fmaf(nshz, xs[r], y[jh][r])));
+                    accg[jl][r] = 0.f;
+                    accg[jh][r] = 0.f;
+                }
+            }
+            xs = v4f{0.f, 0.f, 0.f, 0.f};
+        }
+        // Nothing of the next stage may move above this point: its LDS stores wait for its global loads, which
+        // were issued at the top of this stage and need this stage's compute time to arrive.
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // stages alternate between the PD register sets; nst is even, PD is 1 or 2
+#pragma unroll 1
+    for (int st = 0; st < nst; st += 2) {
+        stage_body(st, sa);
+        if constexpr (PD == 2) stage_body(st + 1, sb);
+        else stage_body(st + 1, sa);
+    }
+
+    // ---- store: lane (word column li, quarter kb) holds tokens 4*kb + r for its 8 channels
+    const int splits = gridDim.x / tiles_n;
+    const int n = 8 * cw;
+    auto finish8 = [&](const float* v, int m, int nn) __attribute__((always_inline)) {  // 8 channels -> fp16 (+ bias), one 16-byte store
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float lo = v[2 * j], hi = v[2 * j + 1];
+            if (bias) {
+                lo = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(lo)) + Lo<LLMQ_F16>::to_f32(bias[nn + 2 * j]);
+                hi = Lo<LLMQ_F16>::to_f32(Lo<LLMQ_F16>::from_f32(hi)) + Lo<LLMQ_F16>::to_f32(bias[nn + 2 * j + 1]);
+            }
+            o[j] = (uint32_t)Lo<LLMQ_F16>::from_f32(lo) | ((uint32_t)Lo<LLMQ_F16>::from_f32(hi) << 16);
+        }
+        *reinterpret_cast<uint4*>(out + (int64_t)m * N + nn) = make_uint4(o[0], o[1], o[2], o[3]);
+    };
+    if (splits == 1) {
+        if (!col_ok) return;
+#pragma unroll
+        for (int r = 0; r < RM; r++) {
+            const int m = 4 * kb + r;
+            if (m >= M) continue;
+            const float v[8] = {y[0][r], y[1][r], y[2][r], y[3][r], y[4][r], y[5][r], y[6][r], y[7][r]};
+            finish8(v, m, n);
+        }
+        return;
+    }
+    constexpr int TILE_CH = SEGW * 8;  // channels per tile
+    float* ptile = reinterpret_cast<float*>(&lds[0][0]);  // [M][TILE_CH] fp32, reuses the weight stages
+    static_assert(2 * kStageRows * STRIDE >= 16 * TILE_CH, "the partial tile fits in the weight stages");
+    __syncthreads();  // every wavefront is done reading the last stage
+#pragma unroll
+    for (int r = 0; r < RM; r++) {
+        const int m = 4 * kb + r;
+        if (m >= M) continue;
+        float4* dst = reinterpret_cast<float4*>(ptile + m * TILE_CH + (16 * wave + li) * 8);
+        dst[0] = make_float4(y[0][r], y[1][r], y[2][r], y[3][r]);
+        dst[1] = make_float4(y[4][r], y[5][r], y[6][r], y[7][r]);
+    }
+    __syncthreads();
+    finish_split_tile<TILE_CH, NT>(ptile, M, N, tile, ks, splits, partials, tickets, bias, out);
+}
+
+inline int cdiv_d(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+}  // namespace
+
+bool awq_decode_supported(int64_t M, int64_t N, int64_t K, int64_t group) {
+    return M >= 1 && M <= 16 && group == kGroup && (N % 32) == 0 && (K % kGroup) == 0 && N / 256 <= kTicketRing / kTicketStride;
+}
+
+// Column tile width (CS wavefronts = 16*CS words), prefetch depth and K split.  Measured on the Qwen2-7B shapes:
+// 128-byte row segments (CS = 2) with one stage in flight beat the wider tile and the deeper prefetch everywhere;
+// about 2048 wavefronts fill the chip, but a block should keep at least two groups (pipeline fill), a column tile
+// at most ~40 arrivals (its ticket is one memory word: arrivals serialize at ~50 ns each), and the fp32 partial
+// sums, written through and read back coherently, at most an eighth of the weight bytes.
+AwqDecodePlan make_awq_decode_plan(int64_t M, int64_t N, int64_t K, int force_cs, int force_pd, int force_splits) {
+    const int groups = (int)(K / kGroup), Nw = (int)(N / 8);
+    AwqDecodePlan p;
+    p.cs = force_cs > 0 ? force_cs : 2;
+    const int strips = cdiv_d(Nw, 16);  // wavefront-wide column strips
+    int s = cdiv_d(2048, strips);
+    if (s > 40) s = 40;
+    if (s > groups / 2) s = groups / 2;
+    if (s > K / (128 * M)) s = (int)(K / (128 * M));  // 2 * S * M * N * 4 <= K * N / 2 / 8
+    if (force_splits > 0) s = force_splits;
+    if (s > groups) s = groups;
+    if (s < 1) s = 1;
+    p.groups_per_block = cdiv_d(groups, s);
+    p.splits = cdiv_d(groups, p.groups_per_block);
+    p.pd = force_pd > 0 ? force_pd : 1;
+    return p;
+}
+
+// fp32 partial sums [splits][M][N]
+size_t awq_decode_workspace_bytes(const AwqDecodePlan& p, int64_t M, int64_t N) {
+    return p.splits > 1 ? (size_t)p.splits * M * N * sizeof(float) : 0;
+}
+
+// Arrival tickets: a ring of counters, all zero between calls (each returns to zero with its last arrival).  A call
+// takes tiles_n consecutive slots at a cursor that only moves forward, so two calls can only meet on a slot if more
+// than kTicketRing / tiles_n later calls were issued while the first had still not run.  One copy per GPU.
+static __device__ unsigned int g_ticket_ring[kTicketRing];
+static unsigned int* g_ticket_ptr[64] = {};  // device address of each GPU's copy, looked up once per device
+
+static int ticket_slots(int tiles_n, unsigned int** out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LLMQ_ERR_LAUNCH;
+    if (!g_ticket_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_ticket_ring)) != hipSuccess || !p) return LLMQ_ERR_LAUNCH;
+        g_ticket_ptr[dev] = static_cast<unsigned int*>(p);  // benign if two threads race: same address
+    }
+    static std::atomic<unsigned long long> cursor{0};
+    unsigned long long at = cursor.fetch_add((unsigned long long)tiles_n * kTicketStride, std::memory_order_relaxed) % kTicketRing;
+    if (at + (unsigned long long)tiles_n * kTicketStride > kTicketRing) at = 0;  // a run that would cross the end starts over at the front
+    *out = g_ticket_ptr[dev] + at;
+    return LLMQ_OK;
+}
+
+int launch_awq_decode(const AwqDecodePlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
+                      const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K,
+                      hipStream_t st) {
+    const int tiles_n = cdiv_d(N / 8, 16 * p.cs);
+    const dim3 grid((unsigned)(tiles_n * p.splits));
+    unsigned int* tickets = nullptr;
+    if (p.splits > 1) {
+        const int rc = ticket_slots(tiles_n, &tickets);
+        if (rc != LLMQ_OK) return rc;
+    }
+#define LLMQ_DECODE_RM(CS_, PD_, RM_)                                                                                 \
+    hipLaunchKernelGGL((awq_decode_kernel<CS_, PD_, RM_>), grid, dim3(CS_ * kWave), 0, st, x, ldx, qw, scales, qz, bias, \
+                       out, ws, tickets, M, N, K, p.groups_per_block, tiles_n)
+#define LLMQ_DECODE(CS_, PD_)                  \
+    do {                                       \
+        if (M == 1) LLMQ_DECODE_RM(CS_, PD_, 1);      \
+        else if (M == 2) LLMQ_DECODE_RM(CS_, PD_, 2); \
+        else LLMQ_DECODE_RM(CS_, PD_, 4);             \
+    } while (0)
+    if (p.cs == 4 && p.pd == 2) LLMQ_DECODE(4, 2);
+    else if (p.cs == 4) LLMQ_DECODE(4, 1);
+    else if (p.pd == 2) LLMQ_DECODE(2, 2);
+    else LLMQ_DECODE(2, 1);
+#undef LLMQ_DECODE
+#undef LLMQ_DECODE_RM
+    return launch_status();
+}
+
+}  // namespace llmq

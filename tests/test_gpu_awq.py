@@ -142,7 +142,7 @@ def test_module_paths_agree_around_the_token_threshold(cuda, K):
 @pytest.fixture
 def force_awq_plan():
     from llmqrt_amd import _abi
-    yield lambda v, splits: _abi.check(_abi.lib().llmq_awq_force_plan(v, splits, 0), "llmq_awq_force_plan")
+    yield lambda v, splits, k_waves=0: _abi.check(_abi.lib().llmq_awq_force_plan(v, splits, k_waves), "llmq_awq_force_plan")
     _abi.lib().llmq_awq_force_plan(0, 0, 0)
 
 
@@ -205,3 +205,52 @@ def test_streaming_kernel_with_shared_unpack(cuda, force_awq_plan, variant, spli
     out = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8,
                           bias=None if bias is None else bias.to(cuda))
     assert rel_err(out, ref) <= REL_TOL, (variant, splits, M, K, N)
+
+
+# (M, K, N): one partial tile (N = 32), tiles that end inside a block's column range (N = 96, 4864 with 256-byte
+# tiles), one group / one stage pair, several groups per block and per split, a strided activation matrix
+DECODE_SHAPES = [(1, 128, 32), (3, 256, 96), (16, 896, 4864), (4, 3584, 4608), (13, 1024, 1056), (2, 2048, 512)]
+
+
+@pytest.mark.parametrize("variant", [8, 9, 10, 11])
+@pytest.mark.parametrize("splits", [0, 1, 3])
+@pytest.mark.parametrize("M,K,N", DECODE_SHAPES)
+def test_decode_kernel_every_variant_and_split(cuda, force_awq_plan, variant, splits, M, K, N):
+    """The LDS-staged decode kernel (up to 16 tokens, group 128): both tile widths (128 / 256 bytes per row,
+    variants 8, 10 / 9, 11), both prefetch depths (variants 10, 11: two stages in flight), fused and split along K,
+    against the oracle; deterministic; a row stride larger than K."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    qw, qz, s = W.awq_weights(N, K, 13 * M + N)
+    x = W.activations(M, 2 * K, 14 * M + K, dtype=torch.float16, outliers=False)[:, :K]  # row stride 2K
+    bias = (0.1 * torch.randn(N, generator=torch.Generator().manual_seed(M))).half() if splits != 1 else None
+    ref = R.awq_gemm(x, qw, qz, s, 128)
+    if bias is not None:
+        ref = (ref.float() + bias.float()).half()
+    force_awq_plan(variant, splits)
+    xd = W.activations(M, 2 * K, 14 * M + K, dtype=torch.float16, outliers=False).to(cuda)[:, :K]
+    assert xd.stride(0) == 2 * K
+    args = (xd, qw.to(cuda), s.to(cuda), qz.to(cuda))
+    out = awq_gemm_triton(*args, split_k_iters=8, bias=None if bias is None else bias.to(cuda))
+    assert out.shape == (M, N) and out.dtype == torch.float16
+    assert rel_err(out, ref) <= REL_TOL, (variant, splits, M, K, N)
+    out2 = awq_gemm_triton(*args, split_k_iters=8, bias=None if bias is None else bias.to(cuda))
+    assert torch.equal(out, out2), "deterministic"
+
+
+def test_decode_kernel_extreme_nibbles_and_zero_tokens(cuda, force_awq_plan):
+    """All-15 weights against zero points 0 and all-0 weights against zero points 15 (the largest |q - z|), and a
+    token block whose rows past M must not leak into the result."""
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    K, N, M = 256, 64, 5
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(M, K, generator=g).half()
+    s = (torch.rand(K // 128, N, generator=g) * 0.02 + 0.001).half()
+    for qv, zv in ((15, 0), (0, 15)):
+        qw = R.awq_pack(torch.full((K, N), qv, dtype=torch.int32))
+        qz = R.awq_pack(torch.full((K // 128, N), zv, dtype=torch.int32))
+        ref = R.awq_gemm(x, qw, qz, s, 128)
+        for variant in (8, 9):
+            force_awq_plan(variant, 0)
+            out = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8)
+            assert rel_err(out, ref) <= REL_TOL, (qv, zv, variant)
