@@ -76,6 +76,13 @@ int llmq_quant_fp8_static(const void* x, int x_dtype, int64_t M, int64_t K, int6
                           uint8_t* q, const float* scale, int scale_is_f32_tensor,
                           llmq_stream_t stream);
 
+/* Replaces quantize_weight_per_channel_absmax, utils/quantization_utils.py:27-38 (the offline weight
+ * quantizer behind SqW8A8BBF16OBF16PerChannel.from_float).  w: [N, K] bf16 / f16 / f32, row stride ldw, any K;
+ * q: int8 [N, K] contiguous; scale: [N] in w_dtype = absmax / 127 without a floor (an all-zero row quantizes
+ * to zeros with a NaN scale, as in the reference).  Arithmetic in w_dtype, as the reference's tensor ops on the GPU. */
+int llmq_quant_i8_weight_per_channel(const void* w, int w_dtype, int64_t N, int64_t K, int64_t ldw,
+                                     int8_t* q, void* scale, llmq_stream_t stream);
+
 size_t llmq_quant_workspace_bytes(void);
 
 /* ------------------------------------------------------------------------------------

@@ -25,6 +25,7 @@ SIGNATURES = {
     "llmq_abi_version": (_int, []),
     "llmq_status_string": (ctypes.c_char_p, [_int]),
     "llmq_quant_i8_per_token": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _int, _vp]),
+    "llmq_quant_i8_weight_per_channel": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "llmq_quant_i8_per_tensor": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _int, _vp, _sz, _vp]),
     "llmq_quant_fp8_per_token": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "llmq_quant_fp8_per_tensor": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),

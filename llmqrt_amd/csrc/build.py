@@ -15,7 +15,7 @@ ROOT = HERE.parent.parent
 OUT_DIR = HERE.parent / "lib"
 OBJ_DIR = OUT_DIR / "obj"
 LIB = OUT_DIR / "libllmq_gfx950.so"
-SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "awq.hip", "awq_decode.hip", "awq_tile.hip"]
+SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "gemm_skinny.hip", "awq.hip", "awq_decode.hip", "awq_tile.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -377,6 +377,48 @@ int per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, vo
     return dispatch_rows<MODE, SCALE_TENSOR>(x, x_dtype, M, K, ldx, q, scale, scale_dtype, partials, nblk, 0, st);
 }
 
+// Per-output-channel int8 weight quantizer (an offline step: one pass when a module is built).  One block per
+// row of W [N, K]; any K, any 16-bit or fp32 dtype; arithmetic in the dtype of W as the reference's tensor ops do on
+// the GPU: scale = round_dt(absmax / 127) with no floor (an all-zero row gives 0 / 0 = NaN, which narrows to 0),
+// q = clamp(rint(round_dt(w / scale)), -128, 127), true division.
+template <int DT>
+__device__ __forceinline__ float wq_load(const void* w, int64_t i) {
+    if (DT == LLMQ_F32) return reinterpret_cast<const float*>(w)[i];
+    return Lo<DT == LLMQ_F32 ? LLMQ_BF16 : DT>::to_f32(reinterpret_cast<const uint16_t*>(w)[i]);
+}
+template <int DT>
+__device__ __forceinline__ float wq_round(float v) {
+    if (DT == LLMQ_F32) return v;
+    return Lo<DT == LLMQ_F32 ? LLMQ_BF16 : DT>::round(v);
+}
+template <int DT>
+__global__ __launch_bounds__(kThreads) void quant_weight_rows_kernel(const void* __restrict__ w, int64_t ldw, int64_t K,
+                                                                      int8_t* __restrict__ q, void* __restrict__ scale_out) {
+    __shared__ float smem[kNW];
+    const int64_t row = blockIdx.x;
+    float amax = 0.f;
+    bool has_nan = false;
+    for (int64_t k = threadIdx.x; k < K; k += kThreads) {
+        const float v = wq_load<DT>(w, row * ldw + k);
+        has_nan |= (v != v);
+        amax = fmaxf(amax, fabsf(v));
+    }
+    if (has_nan) amax = __builtin_nanf("");  // torch's max propagates NaN
+    float m = block_max<kNW>(has_nan ? __builtin_inff() : amax, smem);
+    const float any_nan = block_max<kNW>(has_nan ? 1.f : 0.f, smem);
+    if (any_nan > 0.f) m = __builtin_nanf("");
+    const float s = wq_round<DT>(m / 127.f);
+    if (threadIdx.x == 0) {
+        if (DT == LLMQ_F32) reinterpret_cast<float*>(scale_out)[row] = s;
+        else reinterpret_cast<uint16_t*>(scale_out)[row] = Lo<DT == LLMQ_F32 ? LLMQ_BF16 : DT>::from_f32(s);
+    }
+    for (int64_t k = threadIdx.x; k < K; k += kThreads) {
+        const float t = wq_round<DT>(wq_load<DT>(w, row * ldw + k) / s);
+        const float r = __builtin_rintf(t);
+        q[row * K + k] = (t != t) ? (int8_t)0 : (int8_t)__builtin_amdgcn_fmed3f(r, -128.f, 127.f);
+    }
+}
+
 }  // namespace
 }  // namespace llmq
 
@@ -439,6 +481,21 @@ extern "C" int llmq_quant_fp8_static(const void* x, int x_dtype, int64_t M, int6
     if (!scale) return LLMQ_ERR_NULL;
     return dispatch_rows<MODE_F8, SCALE_STATIC>(x, x_dtype, M, K, ldx, q, nullptr, LLMQ_F32, scale, 1,
                                                 scale_is_f32_tensor ? 1 : 0, (hipStream_t)stream);
+}
+
+extern "C" int llmq_quant_i8_weight_per_channel(const void* w, int w_dtype, int64_t N, int64_t K, int64_t ldw,
+                                                int8_t* q, void* scale, llmq_stream_t stream) {
+    if (w_dtype != LLMQ_BF16 && w_dtype != LLMQ_F16 && w_dtype != LLMQ_F32) return LLMQ_ERR_DTYPE;
+    if (N < 0 || K < 0 || ldw < K || N > 0x7fffffffLL) return LLMQ_ERR_SHAPE;
+    if (N == 0) return LLMQ_OK;
+    if (K == 0) return LLMQ_ERR_SHAPE;
+    if (!w || !q || !scale) return LLMQ_ERR_NULL;
+    const dim3 grid((unsigned)N), block(kThreads);
+    hipStream_t st = (hipStream_t)stream;
+    if (w_dtype == LLMQ_BF16) hipLaunchKernelGGL((quant_weight_rows_kernel<LLMQ_BF16>), grid, block, 0, st, w, ldw, K, q, scale);
+    else if (w_dtype == LLMQ_F16) hipLaunchKernelGGL((quant_weight_rows_kernel<LLMQ_F16>), grid, block, 0, st, w, ldw, K, q, scale);
+    else hipLaunchKernelGGL((quant_weight_rows_kernel<LLMQ_F32>), grid, block, 0, st, w, ldw, K, q, scale);
+    return launch_status();
 }
 
 extern "C" int llmq_rmsnorm(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, const void* weight,

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import torch
 
-from ..quantize import (quantize_activation_per_tensor_absmax,
+from ..quantize import (quantize_activation_per_tensor_absmax, quantize_weight_per_channel_absmax,
                         quantize_activation_per_token_absmax,
                         quantize_activation_per_token_absmax_f32)
 from ..sq_fp8_kernels import (w8a8_int8_linear_bbf16_obf16_per_channel,
@@ -132,8 +132,12 @@ class SqW8A8BBF16OBF16PerChannel(LinearBase):
         if init_only:
             return sq_linear
         w = module.weight.data.float()
-        scale = w.abs().max(dim=1).values / 127          # utils/quantization_utils.py:27-38
-        sq_linear.qweight = (w / scale.view(-1, 1)).round().clamp(-128, 127).to(torch.int8)
+        if w.is_cuda:
+            sq_linear.qweight, scale = quantize_weight_per_channel_absmax(w)   # utils/quantization_utils.py:27-38
+            scale = scale.view(-1)
+        else:  # a module assembled on the host: the same arithmetic in torch
+            scale = w.abs().max(dim=1).values / 127
+            sq_linear.qweight = (w / scale.view(-1, 1)).round().clamp(-128, 127).to(torch.int8)
         sq_linear.weight_scale = scale.float()
         if module.bias is not None:
             sq_linear.bias = module.bias.data.to(dtype)

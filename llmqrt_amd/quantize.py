@@ -123,3 +123,20 @@ def static_per_tensor_quantize(tensor: torch.Tensor, scale) -> torch.Tensor:
         x.data_ptr(), _abi.dtype_code(x.dtype), M, K, x.stride(0) if M > 1 else K, q.data_ptr(),
         sdev.data_ptr(), int(promote), _abi.stream_of(x)), "llmq_quant_fp8_static")
     return q.view(*tensor.shape)
+
+
+@torch.no_grad()
+def quantize_weight_per_channel_absmax(w: torch.Tensor):
+    """Replaces quantize_weight_per_channel_absmax (utils/quantization_utils.py:27-38): w [N, K] bf16 / fp16 / fp32 on
+    the GPU -> (int8 [N, K], scales [N, 1] in w.dtype).  Unlike the reference it leaves w untouched."""
+    assert w.dim() == 2 and w.is_cuda and w.dtype in (torch.bfloat16, torch.float16, torch.float32)
+    if w.stride(1) != 1:
+        w = w.contiguous()
+    N, K = w.shape
+    q = torch.empty((N, K), dtype=torch.int8, device=w.device)
+    scale = torch.empty((N, 1), dtype=w.dtype, device=w.device)
+    if N:
+        _abi.check(_abi.lib().llmq_quant_i8_weight_per_channel(
+            w.data_ptr(), _abi.dtype_code(w.dtype), N, K, w.stride(0), q.data_ptr(), scale.data_ptr(),
+            _abi.stream_of(w)), "llmq_quant_i8_weight_per_channel")
+    return q, scale

@@ -61,9 +61,14 @@ def quantize_activation_per_tensor_absmax(t: torch.Tensor):
 
 
 @torch.no_grad()
-def quantize_weight_per_channel_absmax(w: torch.Tensor):
-    """utils/quantization_utils.py:27-38 (fp32 weights [N, K] -> int8 [N, K], scales [N, 1])."""
-    w = w.float()
+def quantize_weight_per_channel_absmax(w: torch.Tensor, native_dtype: bool = False):
+    """utils/quantization_utils.py:27-38 (weights [N, K] -> int8 [N, K], scales [N, 1]).
+
+    native_dtype=False: fp32 arithmetic (what a module built from fp32 master weights sees).  native_dtype=True: every
+    tensor op in ``w.dtype``, as the reference's ops run on a GPU tensor (scale = absmax / 127 and w / scale each rounded
+    to w.dtype, true division, no floor on the scale; the quotient is then rounded half-to-even and clamped)."""
+    if not native_dtype:
+        w = w.float()
     scale = (w.abs().max(dim=1).values / 127).view(-1, 1)
     q = (w / scale).round().clamp(-128, 127).to(torch.int8)
     return q, scale

@@ -312,12 +312,12 @@ def test_fast_epilogue_is_bit_identical_to_the_general_one(cuda, force_plan, out
 
 
 def test_hip_graph_replays_match_eager(cuda):
-    """The C ABI allocates nothing and launches on the stream it is given, so a decode-sized linear (quantizer +
-    split-K GEMM + its reduction kernel) can be captured into a HIP graph.  Every replay, with fresh inputs
-    and eager work of the same ops in between, must reproduce the eager result bit for bit."""
+    """The C ABI allocates nothing and launches on the stream it is given, so a linear (quantizer + split-K GEMM + its
+    reduction kernel) can be captured into a HIP graph.  Every replay, with fresh inputs and eager work of the same
+    ops in between, must reproduce the eager result bit for bit."""
     from llmqrt_amd import _abi, workloads as W
     L = _abi.lib()
-    M, K, N = 16, 3584, 4608
+    M, K, N = 80, 3584, 3584
     qw, ws = W.int8_weights(N, K, 501)
     qw, ws = qw.to(cuda), ws.to(cuda)
     x = W.activations(M, K, 500).to(cuda)
@@ -436,3 +436,53 @@ def test_fp8_full_prefill_size_properties(cuda):
     assert rel_err(fast[rows.to(cuda)], R.fp8_linear_naive(xq[rows], xs[rows], wq, ws, None)) <= REL_TOL
     doubled = cutlass_f8f8bf16_rowwise_sm89(a, b, None, 2 * xsd, wsd, True)
     assert torch.equal(doubled, 2 * fast)
+
+
+# (M, N, K): every token-tile count (1 / 2 / 4 MFMA token tiles), ragged channels (N % 16 != 0, N % 4 != 0), K that is
+# not a multiple of the K step (16-byte tail), K shorter than one step, more wavefronts than K steps
+SKINNY_SHAPES = [(1, 4608, 3584), (5, 72, 48), (16, 200, 1040), (17, 130, 16), (33, 264, 384), (64, 520, 2064), (48, 37, 80)]
+
+
+@pytest.mark.parametrize("variant", range(6))
+@pytest.mark.parametrize("M,N,K", SKINNY_SHAPES)
+def test_skinny_kernel_every_variant(cuda, force_plan, variant, M, N, K):
+    """The few-token streaming kernel (no LDS staging, one launch), forced with 1 / 2 channel tiles per wavefront and
+    4 / 8 / 16 wavefronts per block: int32 accumulators bit-exact, fp32 accumulators and outputs within tolerance,
+    with and without bias, fp16 and bf16 outputs, e5m2 activations."""
+    from llmqrt_amd.sq_fp8_kernels import (cutlass_f8f8bf16_rowwise_sm89, w8a8_int8_linear_bbf16_obf16_per_channel,
+                                           w8a8_int8_linear_bbf16_obf16_per_tensor)
+    force_plan(100 + variant, 1)
+    qx, sx, qw, sw, bias = _int8_problem(M, N, K, 300 + M)
+    acc_ref = R.int8_gemm_exact(qx, qw)
+    dump = torch.empty((M, N), dtype=torch.int32, device=cuda)
+    y = w8a8_int8_linear_bbf16_obf16_per_channel(qx.to(cuda), qw.to(cuda).t(), bias.to(cuda), sx.to(cuda).view(-1, 1),
+                                                 sw.to(cuda).view(1, -1), _acc_dump=dump)
+    assert torch.equal(dump.cpu(), acc_ref), "int32 accumulators must be bit-exact"
+    assert rel_err(y, R.w8a8_epilogue_per_token_per_channel(acc_ref, sx, sw, bias, torch.bfloat16)) <= REL_TOL
+    y16 = w8a8_int8_linear_bbf16_obf16_per_tensor(qx.to(cuda), qw.to(cuda).t(), bias.half().to(cuda), 1e-3, 0.5)
+    assert y16.dtype == torch.float16
+    assert rel_err(y16, R.w8a8_epilogue_per_tensor(acc_ref, bias.half(), 1e-3, 0.5, torch.float16)) <= REL_TOL
+    xq, xs, wq, ws, fbias = _fp8_problem(M, N, K, 400 + M)
+    facc_ref = R.fp8_gemm_acc(xq, wq)
+    fdump = torch.empty((M, N), dtype=torch.float32, device=cuda)
+    fy = cutlass_f8f8bf16_rowwise_sm89(xq.to(cuda), wq.to(cuda).t(), None, xs.to(cuda), ws.to(cuda).view(1, -1), True,
+                                       _acc_dump=fdump)
+    assert rel_err(fdump, facc_ref) <= FP8_ACC_TOL
+    assert rel_err(fy, R.fp8_epilogue_rowwise(facc_ref, xs, ws, None)) <= REL_TOL
+    x5 = xq.float().to(torch.float8_e5m2)
+    y5 = cutlass_f8f8bf16_rowwise_sm89(x5.to(cuda), wq.to(cuda).t(), fbias.to(cuda), xs.to(cuda), ws.to(cuda).view(1, -1), True)
+    assert rel_err(y5, R.fp8_epilogue_rowwise(R.fp8_gemm_acc(x5, wq), xs, ws, fbias)) <= REL_TOL
+
+
+def test_skinny_kernel_is_deterministic_and_ignores_rows_past_m(cuda):
+    """Default plan at 3 tokens of a strided activation matrix whose following rows hold huge values."""
+    from llmqrt_amd.sq_fp8_kernels import w8a8_int8_linear_bbf16_obf16_per_channel
+    M, N, K = 3, 4608, 3584
+    qx, sx, qw, sw, bias = _int8_problem(M, N, K, 31)
+    big = torch.full((8, K), 127, dtype=torch.int8)
+    big[:M] = qx
+    a = big.to(cuda)[:M]
+    y = w8a8_int8_linear_bbf16_obf16_per_channel(a, qw.to(cuda).t(), bias.to(cuda), sx.to(cuda), sw.to(cuda))
+    y2 = w8a8_int8_linear_bbf16_obf16_per_channel(a, qw.to(cuda).t(), bias.to(cuda), sx.to(cuda), sw.to(cuda))
+    assert torch.equal(y, y2)
+    assert rel_err(y, R.w8a8_epilogue_per_token_per_channel(R.int8_gemm_exact(qx, qw), sx, sw, bias, torch.bfloat16)) <= REL_TOL

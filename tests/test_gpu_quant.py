@@ -150,3 +150,37 @@ def test_full_size_scaling_property(cuda):
     q_ref, s_ref = R.quantize_activation_per_token_absmax(xr)
     q, s = quantize_activation_per_token_absmax(x)
     assert torch.equal(q[rows.to(cuda)].cpu(), q_ref) and torch.equal(s[rows.to(cuda)].cpu().view(torch.int16), s_ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,K", [(64, 264), (3, 7), (1, 3584), (300, 1000)])
+def test_weight_per_channel(cuda, N, K, dtype):
+    """Per-output-channel weight quantizer (utils/quantization_utils.py:27-38) in the dtype of w: codes and scales
+    bit-exact against the oracle, for any K, a strided view, a row far below the activation quantizer's floor and an
+    all-zero row (NaN scale, zero codes)."""
+    from llmqrt_amd.quantize import quantize_weight_per_channel_absmax
+    g = torch.Generator().manual_seed(N * 1000 + K)
+    w = (torch.randn(N, 2 * K, generator=g) * 0.05).to(dtype)
+    w[0] *= 1e-6
+    if N > 2:
+        w[2] = 0
+    wv = w[:, :K]
+    q_ref, s_ref = R.quantize_weight_per_channel_absmax(wv.contiguous(), native_dtype=True)
+    q, s = quantize_weight_per_channel_absmax(w.to(cuda)[:, :K])
+    assert q.dtype == torch.int8 and s.dtype == dtype and s.shape == (N, 1)
+    assert torch.equal(q.cpu(), q_ref)
+    sc, sr = s.cpu().view(-1), s_ref.view(-1)
+    assert torch.equal(torch.isnan(sc), torch.isnan(sr))
+    ok = ~torch.isnan(sr)
+    assert torch.equal(sc[ok], sr[ok])
+
+
+def test_sq_per_channel_module_quantizes_its_weight_on_the_gpu(cuda):
+    """SqW8A8BBF16OBF16PerChannel.from_linear on a GPU module runs the HIP weight quantizer (fp32 arithmetic on the
+    fp32 copy of the weight): buffers equal the oracle's."""
+    from llmqrt_amd.linear import SqW8A8BBF16OBF16PerChannel
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(264, 72, bias=True).to(cuda)
+    mod = SqW8A8BBF16OBF16PerChannel.from_linear(lin, 8, 0, init_only=False, dtype=torch.bfloat16)
+    q_ref, s_ref = R.quantize_weight_per_channel_absmax(lin.weight.data.cpu())
+    assert torch.equal(mod.qweight.cpu(), q_ref) and torch.equal(mod.weight_scale.cpu(), s_ref.view(-1))

@@ -86,6 +86,26 @@ def test_weight_quantizer_argmax_maps_to_127():
 
 
 # ---- e4m3fn ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_weight_quantizer_native_dtype_is_the_per_token_quantizer_without_floor(dtype):
+    """In the dtype of w the per-channel weight quantizer is the per-token activation quantizer (pinned above by known
+    answers, the scalar C restatement and every 16-bit pattern) for every row whose absmax reaches the activation
+    quantizer's floor of 1e-5; below it only the weight quantizer keeps dividing by absmax / 127."""
+    g = torch.Generator().manual_seed(11)
+    w = (torch.randn(64, 264, generator=g) * 0.05).to(dtype)
+    w[3] *= 1e-3
+    w[5, 7] = 3.0
+    q, s = R.quantize_weight_per_channel_absmax(w, native_dtype=True)
+    qt, st = R.quantize_activation_per_token_absmax(w)
+    assert s.dtype == dtype and torch.equal(s.view(-1), st.view(-1)) and torch.equal(q, qt)
+    tiny = (torch.randn(4, 64, generator=g) * 1e-7).to(dtype)
+    q2, s2 = R.quantize_weight_per_channel_absmax(tiny, native_dtype=True)
+    for r in range(4):
+        if tiny[r].abs().max() > 0:
+            assert q2[r].abs().max() >= 126  # the row maximum still maps to the top of the range (the scale is itself rounded)
+    assert R.quantize_activation_per_token_absmax(tiny)[0].abs().max() < 16  # with the floor they stay near zero
+
+
 def test_e4m3_decode_table_matches_format_definition():
     table = json.loads((GOLDEN / "e4m3fn_table.json").read_text())
     c_tab = C.e4m3_decode_table()
