@@ -69,7 +69,7 @@ __device__ __forceinline__ uint16_t to_out(float v, int out_dtype) {
     return out_dtype == LLMQ_BF16 ? Lo<LLMQ_BF16>::from_f32(v) : Lo<LLMQ_F16>::from_f32(v);
 }
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, bool FP8_, int AFMT_ = 0, int RS_ = 2>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, bool FP8_, int AFMT_ = 0, int RS_ = 2, bool DMA_ = false>
 struct GemmCfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
     static constexpr int RS = RS_;                     // K tiles staged in registers: 2, or 1 for fat tiles
@@ -84,10 +84,13 @@ struct GemmCfg {
     static constexpr int KSUB = BK / KB;
     static constexpr int A_LOADS = BM * CPR / NT, B_LOADS = BN * CPR / NT;
     static constexpr int STAGE_CHUNKS = (BM + BN) * CPR;
-    static constexpr size_t LDS_BYTES = 2u * STAGE_CHUNKS * 16u;
+    static constexpr bool DMA = DMA_;                  // operand tiles go global -> LDS directly (global_load_lds), as many LDS stages as fit (up to 4)
+    static constexpr int STAGES = !DMA ? 2 : (4 * STAGE_CHUNKS * 16 <= 160 * 1024 ? (STAGE_CHUNKS * 16 <= 24 * 1024 && BK == 128 ? 3 : 4)
+                                                                                   : (3 * STAGE_CHUNKS * 16 <= 160 * 1024 ? 3 : 2));
+    static constexpr size_t LDS_BYTES = (size_t)STAGES * STAGE_CHUNKS * 16u;
     // Double-buffer the MFMA operand fragments (software pipeline LDS reads under MFMAs).  The fp8
     // fragments are twice as wide; with two wavefronts per SIMD (256 registers each) they do not fit twice.
-    static constexpr bool PIPE = !(FP8 && NT > 256) && !(RS == 1 && NT > 256);
+    static constexpr bool PIPE = DMA || (!(FP8 && NT > 256) && !(RS == 1 && NT > 256));
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be 32-aligned");
     static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "tile must split evenly over threads");
     static_assert(CPR == 4 || CPR == 8, "BK must be 64 or 128");
@@ -317,7 +320,74 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     // ---- main loop: tile kt is computed from LDS stage kt & 1 while tile kt+1 sits in registers
     // and tile kt+2 is in flight from global memory.  Two tiles per iteration, no conditional
     // compute: an odd tile count is padded with a zero tile -----------------------------------
-    if constexpr (C::RS == 2) {
+    if constexpr (C::DMA) {
+        // Operand tiles travel global -> LDS without passing through registers (global_load_lds_dwordx4: each lane
+        // names its own 16 global bytes, a wavefront's 64 pieces land back to back in LDS).  The LDS position is
+        // therefore fixed by the lane and the swizzle is applied on the fetch side: the thread whose piece lands in
+        // chunk slot c' of row r fetches global chunk c' ^ swizzle(r).  With NS LDS stages tile kt is computed while
+        // kt+1 .. kt+NS-1 are in flight; every wait is a counted s_waitcnt on the wavefront's own loads, followed by
+        // the block barrier that publishes the stage.  The loads are issued from assembly so that the compiler,
+        // which would wait for every outstanding load before any later LDS read, does not see them.
+        static_assert(C::KSUB % 2 == 0 && C::KSUB >= 2, "fragment parity must return to 0 at every tile");
+        static_assert(KFULL, "the direct loads cannot zero a ragged K tail");
+        constexpr int LPT = C::A_LOADS + C::B_LOADS;  // loads per thread and tile
+        const int swz = (ld_row / (16 / C::CPR)) & (C::CPR - 1);
+        const uint8_t* pa[C::A_LOADS];
+        const uint8_t* pb[C::B_LOADS];
+#pragma unroll
+        for (int i = 0; i < C::A_LOADS; i++) pa[i] = A + (int64_t)m0 * lda + k_begin + a_off[i] + (ld_c ^ swz) * 16;
+#pragma unroll
+        for (int i = 0; i < C::B_LOADS; i++) pb[i] = B + (int64_t)n0 * ldb + k_begin + b_off[i] + (ld_c ^ swz) * 16;
+        const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem_raw);
+        const uint32_t wave_off = (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 1024u;
+        auto issue_tile = [&](int kt, int stage) {
+            const int koff = min(kt, ktiles - 1) * C::BK;  // past the end: the last tile again, into a stage nobody reads
+            const uint32_t sbase = lds_base + (uint32_t)stage * (C::STAGE_CHUNKS * 16u) + wave_off;
+#pragma unroll
+            for (int i = 0; i < C::A_LOADS; i++) {
+                const uint32_t m0v = sbase + (uint32_t)i * (C::NT * 16u);
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0v), "v"(pa[i] + koff) : "memory", "m0");
+            }
+#pragma unroll
+            for (int i = 0; i < C::B_LOADS; i++) {
+                const uint32_t m0v = sbase + (uint32_t)(C::BM * C::CPR * 16) + (uint32_t)i * (C::NT * 16u);
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0v), "v"(pb[i] + koff) : "memory", "m0");
+            }
+        };
+        constexpr int NS = C::STAGES;
+        auto wait_next_tile = [] {  // at most the NS - 2 youngest tiles may still be in flight
+            constexpr int N = (NS - 2) * LPT;
+            static_assert(N < 64, "vmcnt is a 6-bit counter");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+        };
+#pragma unroll
+        for (int t = 0; t < NS - 1; t++) issue_tile(t, t);
+        wait_next_tile();
+        lds_barrier();
+        read_frags(0, 0, fa[0], fb[0]);
+        int stage = 0;
+#pragma unroll 1
+        for (int kt = 0; kt < ktiles; kt++) {
+            const int prev = stage == 0 ? NS - 1 : stage - 1, next = stage == NS - 1 ? 0 : stage + 1;
+            issue_tile(kt + NS - 1, prev);  // the stage of tile kt-1: every wavefront passed the last barrier after reading it
+#pragma unroll
+            for (int ks = 0; ks < C::KSUB - 1; ks++) {
+                read_frags(stage, ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+                mfma_step(fa[ks & 1], fb[ks & 1]);
+                interleave_reads_with_mfma();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            wait_next_tile();  // tile kt+1 has landed
+            lds_barrier();
+            read_frags(next, 0, fa[0], fb[0]);
+            mfma_step(fa[(C::KSUB - 1) & 1], fb[(C::KSUB - 1) & 1]);
+            interleave_reads_with_mfma();
+            __builtin_amdgcn_sched_barrier(0);
+            stage = next;
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when it is reused or released
+        lds_barrier();
+    } else if constexpr (C::RS == 2) {
         load_tile(0, ra[0], rb[0]);
         load_tile(1, ra[1], rb[1]);
         store_tile(0, 0, ra[0], rb[0]);
@@ -614,7 +684,7 @@ constexpr TileShape kShapes[] = {
 constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
 
 // Tuning/diagnostic knob (llmq_gemm_force_plan): forces a tile configuration and K split.
-int g_force_cfg = -1, g_force_splits = 1;
+int g_force_cfg = -1, g_force_splits = 1, g_force_dma = -1;  // g_force_dma: 0 = register-staged loop only
 bool plan_override(int& cfg, int& splits) {
     if (g_force_cfg < 0) return false;
     cfg = g_force_cfg;
@@ -703,17 +773,23 @@ int launch_cfg(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, int
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LLMQ_ERR_LAUNCH;
         if (!raised[dev]) {
             if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<C, true>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES) != hipSuccess ||
-                hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<C, false>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES) != hipSuccess)
                 return LLMQ_ERR_LAUNCH;
+            if constexpr (!C::DMA)
+                if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<C, false>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES) != hipSuccess)
+                    return LLMQ_ERR_LAUNCH;
             raised[dev] = true;  // benign if two threads race here: both set the same value
         }
     }
     const int tiles = cdiv(M, C::BM) * cdiv(N, C::BN);
     // every split covers whole K tiles -> the loads need no K predicate
     const bool kfull = (K % C::BK == 0) && (p.k_per_split % C::BK == 0);
-    if (kfull)
+    if constexpr (C::DMA) {
+        if (!kfull) return LLMQ_ERR_SHAPE;  // callers route ragged K to the register-staged kernel
+        hipLaunchKernelGGL((gemm_tile_kernel<C, true>), dim3(tiles, p.splits), dim3(C::NT), C::LDS_BYTES, st, A, lda, B,
+                           ldb, M, N, K, p.k_per_split, ep, out, ldo, acc_dump, ws);
+    } else if (kfull)
         hipLaunchKernelGGL((gemm_tile_kernel<C, true>), dim3(tiles, p.splits), dim3(C::NT), C::LDS_BYTES, st, A, lda, B,
                            ldb, M, N, K, p.k_per_split, ep, out, ldo, acc_dump, ws);
     else
@@ -722,19 +798,30 @@ int launch_cfg(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, int
     return launch_status();
 }
 
+template <bool FP8, int AFMT, bool DMA>
+int launch_shape(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, int M, int N, int K, const Plan& p,
+                 const Epilogue& ep, void* out, int64_t ldo, void* acc_dump, void* ws, hipStream_t st) {
+    switch (p.cfg) {
+        case 0: return launch_cfg<GemmCfg<256, 256, 64, 2, 2, FP8, AFMT, 2, DMA && !FP8>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
+        case 1: return launch_cfg<GemmCfg<256, 256, 64, 2, 4, FP8, AFMT, 2, DMA && !FP8>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
+        case 2: return launch_cfg<GemmCfg<256, 128, 64, 2, 2, FP8, AFMT, 2, DMA && !FP8>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
+        case 3: return launch_cfg<GemmCfg<128, 128, 64, 2, 2, FP8, AFMT, 2, DMA && !FP8>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
+        case 4: return launch_cfg<GemmCfg<64, 128, 128, 2, 2, FP8, AFMT, 2, DMA>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
+        case 6: return launch_cfg<GemmCfg<256, 256, 128, 2, 4, FP8, AFMT, 1, DMA>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
+        default: return launch_cfg<GemmCfg<32, 128, 128, 1, 4, FP8, AFMT, 2, DMA>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
+    }
+}
+
 template <bool FP8, int AFMT>
 int launch_gemm(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, int M, int N, int K, const Plan& p,
                 const Epilogue& ep, void* out, int64_t ldo, void* acc_dump, void* ws, hipStream_t st) {
-    int rc;
-    switch (p.cfg) {
-        case 0: rc = launch_cfg<GemmCfg<256, 256, 64, 2, 2, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
-        case 1: rc = launch_cfg<GemmCfg<256, 256, 64, 2, 4, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
-        case 2: rc = launch_cfg<GemmCfg<256, 128, 64, 2, 2, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
-        case 3: rc = launch_cfg<GemmCfg<128, 128, 64, 2, 2, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
-        case 4: rc = launch_cfg<GemmCfg<64, 128, 128, 2, 2, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
-        case 6: rc = launch_cfg<GemmCfg<256, 256, 128, 2, 4, FP8, AFMT, 1>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
-        default: rc = launch_cfg<GemmCfg<32, 128, 128, 1, 4, FP8, AFMT>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st); break;
-    }
+    // Operand tiles go straight into LDS whenever every split covers whole K tiles (the direct loads cannot zero a
+    // ragged tail); llmq_gemm_force_plan(cfg | 64, .) keeps the register-staged loop.  The fp8 K step is 64 bytes, so
+    // the 64-byte K tiles have a single sub-step there and stay register-staged.
+    const int bk = kShapes[p.cfg].bk;
+    const bool dma = g_force_dma != 0 && K % bk == 0 && p.k_per_split % bk == 0;
+    int rc = dma ? launch_shape<FP8, AFMT, true>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st)
+                 : launch_shape<FP8, AFMT, false>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
     if (rc != LLMQ_OK || p.splits == 1) return rc;
     const int64_t total = (int64_t)M * N;
     const int blocks = (int)std::min<int64_t>((total + 255) / 256, 4096);
@@ -765,6 +852,8 @@ int gemm_entry(bool fp8, int a_format, const uint8_t* A, int64_t lda, const uint
     Plan p = make_plan(M, N, K);
     // fp8 fragments are twice as wide: the 8-wave prefill tile runs ~5 % faster with 128-byte K tiles
     if (fp8 && g_force_cfg < 0 && p.cfg == 1 && p.splits == 1) p.cfg = 6;
+    // int8 with direct loads: no staging registers, so the 128-byte K tile fits (half the barriers, whole lines per row)
+    if (!fp8 && g_force_cfg < 0 && p.cfg == 1 && K % 128 == 0 && p.k_per_split % 128 == 0) p.cfg = 6;
     if (p.splits > 1) {
         if (!ws || ws_bytes < (size_t)p.splits * M * N * 4) return LLMQ_ERR_WORKSPACE;
     }
@@ -820,7 +909,10 @@ extern "C" int llmq_gemm_w8a8_static(const int8_t* A, int64_t lda, const int8_t*
 }
 
 extern "C" int llmq_gemm_force_plan(int cfg, int splits) {
+    int dma = -1;
+    if (cfg >= 0 && cfg < 100 && (cfg & 64)) dma = 0, cfg &= ~64;
     if ((cfg >= kNumShapes && (cfg < 100 || cfg > 105)) || splits < 1 || splits > 64) return LLMQ_ERR_SHAPE;
+    g_force_dma = dma;
     g_force_cfg = cfg;
     g_force_splits = splits;
     return LLMQ_OK;

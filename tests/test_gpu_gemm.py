@@ -66,8 +66,9 @@ def test_w8a8_per_channel(cuda, M, N, K):
     assert rel_err(y, naive) <= REL_TOL
 
 
-# K = 1040 gives an odd number of K tiles plus a 16-byte tail, 1024 an even number, 128 / 64 a single tile
-@pytest.mark.parametrize("K", [1040, 1024, 128, 64, 384])
+# K = 1040 gives an odd number of K tiles plus a 16-byte tail, 1024 an even number, 128 / 64 a single tile,
+# 2560 more tiles than LDS stages of the direct-load loop
+@pytest.mark.parametrize("K", [1040, 1024, 128, 64, 384, 2560])
 @pytest.mark.parametrize("splits", [1, 2, 3])
 def test_w8a8_every_tile_config(cuda, force_plan, splits, K):
     """Each tile configuration and the split-K path, on a ragged shape; accumulators bit-exact."""
@@ -76,7 +77,8 @@ def test_w8a8_every_tile_config(cuda, force_plan, splits, K):
     qx, sx, qw, sw, bias = _int8_problem(M, N, K, 7)
     acc_ref = R.int8_gemm_exact(qx, qw)
     y_ref = R.w8a8_epilogue_per_token_per_channel(acc_ref, sx, sw, bias, torch.bfloat16)
-    for cfg in range(_num_cfgs()):
+    # cfg: operand tiles loaded straight into LDS where K allows; cfg | 64: the register-staged loop
+    for cfg in [c | off for c in range(_num_cfgs()) for off in (0, 64)]:
         force_plan(cfg, splits)
         dump = torch.empty((M, N), dtype=torch.int32, device=cuda)
         y = w8a8_int8_linear_bbf16_obf16_per_channel(qx.to(cuda), qw.to(cuda).t(), bias.to(cuda), sx.to(cuda),
@@ -171,7 +173,7 @@ def test_fp8_rowwise(cuda, M, N, K):
     assert rel_err(y_nb, R.fp8_epilogue_rowwise(acc_ref, xs, ws, None)) <= REL_TOL
 
 
-@pytest.mark.parametrize("K", [1040, 1024, 128, 64, 384])
+@pytest.mark.parametrize("K", [1040, 1024, 128, 64, 384, 2560])
 @pytest.mark.parametrize("splits", [1, 2, 3])
 def test_fp8_every_tile_config(cuda, force_plan, splits, K):
     from llmqrt_amd.sq_fp8_kernels import cutlass_f8f8bf16_rowwise_sm89
@@ -179,7 +181,7 @@ def test_fp8_every_tile_config(cuda, force_plan, splits, K):
     xq, xs, wq, ws, bias = _fp8_problem(M, N, K, 9)
     acc_ref = R.fp8_gemm_acc(xq, wq)
     y_ref = R.fp8_epilogue_rowwise(acc_ref, xs, ws, bias)
-    for cfg in range(_num_cfgs()):
+    for cfg in [c | off for c in range(_num_cfgs()) for off in (0, 64)]:
         force_plan(cfg, splits)
         dump = torch.empty((M, N), dtype=torch.float32, device=cuda)
         y = cutlass_f8f8bf16_rowwise_sm89(xq.to(cuda), wq.to(cuda).t(), bias.to(cuda), xs.to(cuda),
