@@ -174,6 +174,15 @@ int llmq_gemm_w8a8_static(const int8_t* A, int64_t lda, const int8_t* B, int64_t
                           int64_t M, int64_t N, int64_t K, llmq_stream_t stream);
 size_t llmq_gemm_static_scratch_bytes(void);
 
+/* fp16 GEMM with fp32 accumulation, out = alpha * A B^T + beta * bias: replaces the torch.matmul of the reference's
+ * many-token AWQ path (nn_models/modules/linear/linear_awq.py:51-53) after llmq_awq_dequant_t.  A: fp16 [M, K], B: fp16
+ * [N, K] (both K-contiguous, K % 8 == 0, lda % 8 == 0, ldb % 8 == 0, 16-byte aligned); bias: [N] or null; out: bf16 / f16
+ * [M, N].  Same tile kernels, plans and workspace rule as llmq_gemm_w8a8 (llmq_gemm_f16_workspace_bytes). */
+int llmq_gemm_f16(const void* A, int64_t lda, const void* B, int64_t ldb, float alpha, const void* bias, int bias_dtype,
+                  float beta, void* out, int out_dtype, int64_t ldo, int64_t M, int64_t N, int64_t K, float* acc_dump,
+                  void* workspace, size_t workspace_bytes, llmq_stream_t stream);
+size_t llmq_gemm_f16_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
 /* Tuning / test hook with no counterpart in the reference: force tile configuration `cfg`
  * (0 .. llmq_gemm_num_configs()-1) and K split `splits` for every later GEMM call of this
  * process; cfg < 0 restores the built-in heuristic.  Process-global, not thread-safe. */
@@ -215,6 +224,12 @@ int llmq_awq_force_plan(int v, int splits, int k_waves);
  * utils/packing_utils.py:65-80 (dequantize_gemm). */
 int llmq_awq_dequant(const int32_t* qweight, const void* scales, const int32_t* qzeros,
                      void* out, int64_t K, int64_t N, int64_t group, llmq_stream_t stream);
+
+/* The same dequantized weights written as the transpose, fp16 [N, K] with K contiguous (the B operand of
+ * llmq_gemm_f16): together they replace awq_dequantize_triton + torch.matmul of the reference's many-token path
+ * (nn_models/modules/linear/linear_awq.py:49-53).  group % 8 == 0. */
+int llmq_awq_dequant_t(const int32_t* qweight, const void* scales, const int32_t* qzeros, void* out,
+                       int64_t K, int64_t N, int64_t group, llmq_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -42,12 +42,15 @@ SIGNATURES = {
     "llmq_gemm_w8a8_static": (_int, [_vp, _i64, _vp, _i64, _vp, _vp, _f32, _vp, _vp, _int, _f32, _vp, _int, _i64,
                                      _i64, _i64, _i64, _vp]),
     "llmq_gemm_static_scratch_bytes": (_sz, []),
+    "llmq_gemm_f16": (_int, [_vp, _i64, _vp, _i64, _f32, _vp, _int, _f32, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _sz, _vp]),
+    "llmq_gemm_f16_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "llmq_gemm_force_plan": (_int, [_int, _int]),
     "llmq_gemm_num_configs": (_int, []),
     "llmq_awq_gemm": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
     "llmq_awq_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "llmq_awq_force_plan": (_int, [_int, _int, _int]),
     "llmq_awq_dequant": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "llmq_awq_dequant_t": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
 }
 
 _lib = None

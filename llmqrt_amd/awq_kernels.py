@@ -39,6 +39,47 @@ def awq_dequantize_triton(qweight: torch.Tensor, scales: torch.Tensor, zeros: to
 
 
 @torch.no_grad()
+def awq_dequantize_transposed(qweight: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor) -> torch.Tensor:
+    """The same dequantized weights as awq_dequantize_triton, written as fp16 [N, K] (K contiguous): the weight operand
+    of ``gemm_f16``.  No counterpart in the reference (its torch.matmul takes the [K, N] tensor)."""
+    K = qweight.shape[0]
+    N = scales.shape[1]
+    group_size = qweight.shape[0] // scales.shape[0]
+    assert K > 0 and N > 0 and group_size % 8 == 0
+    _check_layout(qweight, scales, zeros, K, N, group_size)
+    result = torch.empty(N, K, device=qweight.device, dtype=scales.dtype)
+    _abi.check(_abi.lib().llmq_awq_dequant_t(qweight.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
+                                             result.data_ptr(), K, N, group_size, _abi.stream_of(qweight)),
+               "llmq_awq_dequant_t")
+    return result
+
+
+@torch.no_grad()
+def gemm_f16(x: torch.Tensor, w_nk: torch.Tensor, bias: torch.Tensor | None = None, *, _acc_dump=None) -> torch.Tensor:
+    """x fp16 [M, K] times w_nk^T (fp16 [N, K]) -> fp16 [M, N], fp32 accumulation on the matrix cores (+ bias).
+    Replaces the torch.matmul of the reference's many-token path (linear_awq.py:51-53)."""
+    assert x.dtype == torch.float16 and w_nk.dtype == torch.float16 and x.dim() == 2 and w_nk.dim() == 2
+    assert x.is_cuda and w_nk.device == x.device and x.shape[1] == w_nk.shape[1]
+    M, K = x.shape
+    N = w_nk.shape[0]
+    assert K % 8 == 0
+    if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+        x = x.contiguous()
+    if w_nk.stride(1) != 1 or w_nk.stride(0) % 8 or w_nk.data_ptr() % 16:
+        w_nk = w_nk.contiguous()
+    out = torch.empty((M, N), dtype=torch.float16, device=x.device)
+    if M == 0 or N == 0:
+        return out
+    L = _abi.lib()
+    ws = _abi.workspaces.get(x.device, L.llmq_gemm_f16_workspace_bytes(M, N, K))
+    _abi.check(L.llmq_gemm_f16(x.data_ptr(), x.stride(0), w_nk.data_ptr(), w_nk.stride(0), 1.0, _abi.ptr(bias),
+                               _abi.dtype_code(bias.dtype) if bias is not None else 0, 1.0, out.data_ptr(), _abi.F16, N,
+                               M, N, K, _abi.ptr(_acc_dump), _abi.ptr(ws), ws.numel() if ws is not None else 0,
+                               _abi.stream_of(x)), "llmq_gemm_f16")
+    return out
+
+
+@torch.no_grad()
 def awq_gemm_triton(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, qzeros: torch.Tensor,
                     split_k_iters: int, block_size_m: int = 32, block_size_n: int = 32,
                     block_size_k: int = 32, *, bias: torch.Tensor | None = None) -> torch.Tensor:

@@ -643,6 +643,51 @@ __global__ __launch_bounds__(256) void awq_dequant_rows_kernel(const uint32_t* _
     }
 }
 
+// Dequantizer that writes the transpose, fp16 [N, K] with K contiguous: the operand layout of the MFMA GEMM
+// (llmq_gemm_f16), for the many-token path.  Same arithmetic as awq_dequant_rows_kernel (bit-identical values).  A
+// thread owns 8 consecutive K rows of one word column, i.e. 8 k-values of 8 channels = one 16-byte piece of 8 output
+// rows; the lanes of a wavefront are (k octet, word column) = (lane % 8, lane / 8), so that a store instruction writes
+// 8 channel rows x 128 contiguous bytes, and the 4 wavefronts of a block read the four 32-byte quarters of the same
+// packed 128-byte line.
+__global__ __launch_bounds__(256) void awq_dequant_t_kernel(const uint32_t* __restrict__ qw,
+                                                             const uint16_t* __restrict__ scales,
+                                                             const uint32_t* __restrict__ qz,
+                                                             uint16_t* __restrict__ out, int K, int Nw, int G) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int c = blockIdx.x * 32 + wave * 8 + (lane >> 3);
+    const int k0 = (int)blockIdx.y * 64 + (lane & 7) * 8;
+    if (c >= Nw || k0 >= K) return;
+    const int64_t g = k0 / G;
+    uint32_t w[8];
+#pragma unroll
+    for (int r = 0; r < 8; r++) w[r] = qw[(int64_t)(k0 + r) * Nw + c];
+    const uint32_t z = qz[g * Nw + c];
+    const uint4 sv = *reinterpret_cast<const uint4*>(scales + (g * Nw + c) * 8);
+    const uint32_t sw[4] = {sv.x, sv.y, sv.z, sv.w};
+    uint32_t o[8][4];  // o[r][j]: channels 2j (low half) and 2j + 1 (high half) of row k0 + r
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const h2 zp = __builtin_bit_cast(h2, ((z >> (4 * j)) & 0x000F000Fu) | 0x64006400u);
+        const h2 sp = __builtin_bit_cast(h2, sw[j]);
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+            const h2 q = __builtin_bit_cast(h2, ((w[r] >> (4 * j)) & 0x000F000Fu) | 0x64006400u);
+            o[r][j] = __builtin_bit_cast(uint32_t, (q - zp) * sp);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t sel = h ? 0x07060302u : 0x05040100u;  // the high / low halves of two registers
+            uint32_t v[4];
+#pragma unroll
+            for (int pr = 0; pr < 4; pr++) v[pr] = __builtin_amdgcn_perm(o[2 * pr + 1][j], o[2 * pr][j], sel);
+            *reinterpret_cast<uint4*>(out + (int64_t)(8 * c + 2 * j + h) * K + k0) = make_uint4(v[0], v[1], v[2], v[3]);
+        }
+    }
+}
+
 struct AwqPlan { int v, mt, splits, chunks_per_block; };
 
 inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
@@ -864,5 +909,19 @@ extern "C" int llmq_awq_dequant(const int32_t* qweight, const void* scales, cons
     const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
     hipLaunchKernelGGL(awq_dequant_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const uint32_t*)qweight,
                        (const uint16_t*)scales, (const uint32_t*)qzeros, (uint16_t*)out, K, (int)(N / 8), (int)group);
+    return launch_status();
+}
+
+extern "C" int llmq_awq_dequant_t(const int32_t* qweight, const void* scales, const int32_t* qzeros, void* out,
+                                  int64_t K, int64_t N, int64_t group, llmq_stream_t stream) {
+    if (K < 0 || N < 0) return LLMQ_ERR_SHAPE;
+    if (K == 0 || N == 0) return LLMQ_OK;
+    if (!qweight || !scales || !qzeros || !out) return LLMQ_ERR_NULL;
+    if ((N & 7) || group <= 0 || (K % group) || (group & 7) || N > 0x7fffffffLL || K > 0x7fffffffLL || (K + 63) / 64 > 65535)
+        return LLMQ_ERR_SHAPE;
+    if (!aligned16(scales) || !aligned16(out)) return LLMQ_ERR_ALIGN;
+    const dim3 grid((unsigned)((N / 8 + 31) / 32), (unsigned)((K + 63) / 64));
+    hipLaunchKernelGGL(awq_dequant_t_kernel, grid, dim3(256), 0, (hipStream_t)stream, (const uint32_t*)qweight,
+                       (const uint16_t*)scales, (const uint32_t*)qzeros, (uint16_t*)out, (int)K, (int)(N / 8), (int)group);
     return launch_status();
 }

@@ -49,6 +49,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 constexpr int kNumXcd = 8;
 constexpr int kGroupM = 8;
@@ -74,7 +75,9 @@ struct GemmCfg {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_;
     static constexpr int RS = RS_;                     // K tiles staged in registers: 2, or 1 for fat tiles
     static constexpr bool FP8 = FP8_;
-    static constexpr int AFMT = AFMT_;                 // fp8 A format selector: 0 e4m3, 1 e5m2
+    static constexpr int AFMT = AFMT_;                 // fp8 A format selector: 0 e4m3, 1 e5m2; without FP8: 2 = fp16 operands
+    static constexpr bool F16 = !FP8_ && AFMT_ == 2;   // v_mfma_f32_32x32x16_f16: 16 K-elements = 32 K-bytes per MFMA, like int8
+    static constexpr bool FACC = FP8_ || F16;          // fp32 accumulators
     static constexpr int NT = WM * WN * kWave;
     static constexpr int WTM = BM / WM, WTN = BN / WN; // wavefront tile
     static constexpr int TM = WTM / 32, TN = WTN / 32; // MFMA tiles per wavefront
@@ -120,7 +123,7 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     void* __restrict__ acc_dump, void* __restrict__ partials) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem_raw[];
     uint4* lds = reinterpret_cast<uint4*>(smem_raw);
-    using acc_t = typename std::conditional<C::FP8, v16f, v16i>::type;
+    using acc_t = typename std::conditional<C::FACC, v16f, v16i>::type;
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int wm = wave / C::WN, wn = wave % C::WN;
@@ -238,6 +241,9 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
                 if constexpr (C::FP8)
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[i][j], 0, C::AFMT,
                                                                                 0, 0, 0, 0);
+                else if constexpr (C::F16)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, bf[j]), __builtin_bit_cast(v8h, af[i]),
+                                                                       acc[i][j], 0, 0, 0);
                 else
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
             }
@@ -716,7 +722,8 @@ bool skinny_plan(int64_t M, int64_t N, int64_t K, int& t, int& nw) {
 
 // Pick the tile shape and K split with the smallest modelled time:
 // waves of blocks over the CUs x per-block MFMA time, with a floor from the bytes each block streams.
-Plan make_plan(int64_t M, int64_t N, int64_t K) {
+// mfma_scale: matrix-core time per K byte relative to int8 / fp8 (fp16: 2)
+Plan make_plan(int64_t M, int64_t N, int64_t K, double mfma_scale = 1.0) {
     int ocfg, osp;
     if (plan_override(ocfg, osp) && ocfg < 100) {
         const TileShape s = kShapes[ocfg < kNumShapes ? ocfg : kNumShapes - 1];
@@ -754,8 +761,9 @@ Plan make_plan(int64_t M, int64_t N, int64_t K) {
             if (eff_sp != sp) continue;
             const int64_t slots = (int64_t)kNumCu * md.per_cu, blocks = tiles * sp;
             const int64_t full_rounds = blocks / slots, rest = blocks % slots;
-            double t = full_rounds * (kps / 64.0 * md.t_tile + md.fixed);
-            if (rest) t += kps / 64.0 * md.t_tile * (0.52 + 0.48 * (double)rest / slots) + md.fixed;
+            const double tt = md.t_tile * mfma_scale;
+            double t = full_rounds * (kps / 64.0 * tt + md.fixed);
+            if (rest) t += kps / 64.0 * tt * (0.52 + 0.48 * (double)rest / slots) + md.fixed;
             if (sp > 1) t += 5.0 + (double)M * N * sp * 8.0 / 8.0e6;
             if (t < best_t) { best_t = t; best = Plan{md.cfg, sp, kps}; }
         }
@@ -825,15 +833,17 @@ int launch_gemm(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, in
     if (rc != LLMQ_OK || p.splits == 1) return rc;
     const int64_t total = (int64_t)M * N;
     const int blocks = (int)std::min<int64_t>((total + 255) / 256, 4096);
-    hipLaunchKernelGGL((splitk_epilogue_kernel<FP8>), dim3(blocks), dim3(256), 0, st, ws, p.splits, M, N, ep, out, ldo,
+    hipLaunchKernelGGL((splitk_epilogue_kernel<FP8 || AFMT == 2>), dim3(blocks), dim3(256), 0, st, ws, p.splits, M, N, ep, out, ldo,
                        acc_dump);
     return launch_status();
 }
 
-int gemm_entry(bool fp8, int a_format, const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb,
+// op: 0 int8, 1 fp8 (a_format picks the A format), 2 fp16 (K, lda, ldb in bytes, i.e. twice the element counts)
+int gemm_entry(int op, int a_format, const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb,
                const float* a_scale, const float* w_scale, float alpha, const float* alpha_dev, const void* bias,
                int bias_dtype, float beta, void* out, int out_dtype, int64_t ldo, int64_t M, int64_t N, int64_t K,
                void* acc_dump, void* ws, size_t ws_bytes, hipStream_t st) {
+    const bool fp8 = op == 1;
     if (M < 0 || N < 0 || K < 0) return LLMQ_ERR_SHAPE;
     if (M == 0 || N == 0) return LLMQ_OK;
     if (!A || !B || !out) return LLMQ_ERR_NULL;
@@ -844,12 +854,12 @@ int gemm_entry(bool fp8, int a_format, const uint8_t* A, int64_t lda, const uint
     if (fp8 && a_format != LLMQ_E4M3 && a_format != LLMQ_E5M2) return LLMQ_ERR_DTYPE;
     if (!aligned16(A) || !aligned16(B)) return LLMQ_ERR_ALIGN;
     int sk_t, sk_nw;
-    if (skinny_plan(M, N, K, sk_t, sk_nw)) {
+    if (op != 2 && skinny_plan(M, N, K, sk_t, sk_nw)) {
         const SkinnyEpilogue sep{a_scale, w_scale, alpha_dev, bias, alpha, beta, bias_dtype, out_dtype};
         return launch_gemm_skinny(fp8, a_format == LLMQ_E5M2 ? 1 : 0, sk_t, sk_nw, A, lda, B, ldb, (int)M, (int)N, (int)K, sep,
                                   out, ldo, acc_dump, st);
     }
-    Plan p = make_plan(M, N, K);
+    Plan p = make_plan(M, N, K, op == 2 ? 2.0 : 1.0);
     // fp8 fragments are twice as wide: the 8-wave prefill tile runs ~5 % faster with 128-byte K tiles
     if (fp8 && g_force_cfg < 0 && p.cfg == 1 && p.splits == 1) p.cfg = 6;
     // int8 with direct loads: no staging registers, so the 128-byte K tile fits (half the barriers, whole lines per row)
@@ -858,6 +868,7 @@ int gemm_entry(bool fp8, int a_format, const uint8_t* A, int64_t lda, const uint
         if (!ws || ws_bytes < (size_t)p.splits * M * N * 4) return LLMQ_ERR_WORKSPACE;
     }
     Epilogue ep{a_scale, w_scale, alpha_dev, bias, alpha, beta, bias_dtype, out_dtype};
+    if (op == 2) return launch_gemm<false, 2>(A, lda, B, ldb, (int)M, (int)N, (int)K, p, ep, out, ldo, acc_dump, ws, st);
     if (!fp8) return launch_gemm<false, 0>(A, lda, B, ldb, (int)M, (int)N, (int)K, p, ep, out, ldo, acc_dump, ws, st);
     if (a_format == LLMQ_E4M3)
         return launch_gemm<true, 0>(A, lda, B, ldb, (int)M, (int)N, (int)K, p, ep, out, ldo, acc_dump, ws, st);
@@ -903,7 +914,7 @@ extern "C" int llmq_gemm_w8a8_static(const int8_t* A, int64_t lda, const int8_t*
     void* ws = nullptr;
     const int rc = static_scratch(&ws);
     if (rc != LLMQ_OK) return rc;
-    return gemm_entry(false, 0, (const uint8_t*)A, lda, (const uint8_t*)B, ldb, a_scale, w_scale, alpha, alpha_dev,
+    return gemm_entry(0, 0, (const uint8_t*)A, lda, (const uint8_t*)B, ldb, a_scale, w_scale, alpha, alpha_dev,
                       bias, bias_dtype, beta, out, out_dtype, ldo, M, N, K, nullptr, ws, kStaticScratchBytes,
                       (hipStream_t)stream);
 }
@@ -933,7 +944,7 @@ extern "C" int llmq_gemm_w8a8(const int8_t* A, int64_t lda, const int8_t* B, int
                               int bias_dtype, float beta, void* out, int out_dtype, int64_t ldo, int64_t M, int64_t N,
                               int64_t K, int32_t* acc_dump, void* workspace, size_t workspace_bytes,
                               llmq_stream_t stream) {
-    return gemm_entry(false, 0, (const uint8_t*)A, lda, (const uint8_t*)B, ldb, a_scale, w_scale, alpha, alpha_dev,
+    return gemm_entry(0, 0, (const uint8_t*)A, lda, (const uint8_t*)B, ldb, a_scale, w_scale, alpha, alpha_dev,
                       bias, bias_dtype, beta, out, out_dtype, ldo, M, N, K, acc_dump, workspace, workspace_bytes,
                       (hipStream_t)stream);
 }
@@ -943,6 +954,21 @@ extern "C" int llmq_gemm_fp8(const uint8_t* A, int a_format, int64_t lda, const 
                              const void* bias, int bias_dtype, float beta, void* out, int out_dtype, int64_t ldo,
                              int64_t M, int64_t N, int64_t K, float* acc_dump, void* workspace,
                              size_t workspace_bytes, llmq_stream_t stream) {
-    return gemm_entry(true, a_format, A, lda, B, ldb, a_scale, w_scale, alpha, alpha_dev, bias, bias_dtype, beta, out,
+    return gemm_entry(1, a_format, A, lda, B, ldb, a_scale, w_scale, alpha, alpha_dev, bias, bias_dtype, beta, out,
                       out_dtype, ldo, M, N, K, acc_dump, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" size_t llmq_gemm_f16_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const Plan p = make_plan(M, N, 2 * K, 2.0);
+    return p.splits > 1 ? (size_t)p.splits * M * N * 4 : 0;
+}
+
+extern "C" int llmq_gemm_f16(const void* A, int64_t lda, const void* B, int64_t ldb, float alpha, const void* bias,
+                             int bias_dtype, float beta, void* out, int out_dtype, int64_t ldo, int64_t M, int64_t N,
+                             int64_t K, float* acc_dump, void* workspace, size_t workspace_bytes, llmq_stream_t stream) {
+    if (K < 0 || (K & 7) || (lda & 7) || (ldb & 7)) return LLMQ_ERR_SHAPE;  // 16-byte pieces of fp16
+    return gemm_entry(2, 0, (const uint8_t*)A, 2 * lda, (const uint8_t*)B, 2 * ldb, nullptr, nullptr, alpha, nullptr, bias,
+                      bias_dtype, beta, out, out_dtype, ldo, M, N, 2 * K, acc_dump, workspace, workspace_bytes,
+                      (hipStream_t)stream);
 }

@@ -5,7 +5,7 @@ from __future__ import annotations
 
 import torch
 
-from ..awq_kernels import awq_dequantize_triton, awq_gemm_triton
+from ..awq_kernels import awq_dequantize_transposed, awq_dequantize_triton, awq_gemm_triton, gemm_f16
 from .linear_base import LinearBase
 
 AWQ_ORDER = (0, 2, 4, 6, 1, 3, 5, 7)
@@ -21,20 +21,23 @@ def _pack_rows(values: torch.Tensor, w_bit: int = 4) -> torch.Tensor:
     return torch.where(word >= 2 ** 31, word - 2 ** 32, word).to(torch.int32)
 
 
-# Set to False to keep every token count on this package's own kernels (llmq_awq_gemm) instead of switching to
-# dequantize + torch.matmul for long prompts.
+# Set to False to keep every token count on the fused kernels (llmq_awq_gemm) instead of switching to dequantize +
+# fp16 GEMM for long prompts.
 USE_DEQUANT_MATMUL = True
 
 
-def dequant_matmul_token_threshold(in_features: int) -> int:
-    """Token count from which dequantize + fp16 matmul beats the fused kernels on MI355X.
+def dequant_matmul_token_threshold(in_features: int, out_features: int = 0) -> int:
+    """Token count from which dequantize (transposed, llmq_awq_dequant_t) + fp16 MFMA GEMM (llmq_gemm_f16) beats the
+    fused kernels on MI355X.
 
-    The reference switches at 1024 tokens (linear_awq.py:22,47).  Measured on the Qwen2-7B shapes, the fused
-    path (streaming kernel up to 64 tokens, tile kernel with in-loop dequantization above) is ahead up to
-    ~400 (qkv) to ~560 (gate_up) tokens for K = 3584 and ~900 for K = 18944 (down); beyond that the dequantizer's
-    fixed cost is amortized and the library matmul runs at a higher rate than the tile kernel.  Both paths are
-    within 1e-2 (max relative) of dequantize-then-matmul in fp32."""
-    return 448 if in_features <= 8192 else 896
+    The reference switches to dequantize + torch.matmul at 1024 tokens (linear_awq.py:22,47).  Here both sides are
+    this library's kernels; measured on the Qwen2-7B shapes the fused path (streaming kernels up to 64 tokens, tile
+    kernel with in-loop dequantization above) is ahead up to ~380 tokens for down (K = 18944), ~500-750 for qkv / o
+    and ~1500 for gate_up (N = 37888, where the dequantizer's 70 us take longest to amortize).  Both paths are within
+    1e-2 (max relative) of dequantize-then-matmul in fp32."""
+    if in_features > 8192:
+        return 384
+    return 1536 if out_features > 8192 else 640
 
 
 def awq_linear_forward(x, qweight, qzeros, scales, w_bit=4, group_size=128, bias=None, out_features=0):
@@ -43,10 +46,14 @@ def awq_linear_forward(x, qweight, qzeros, scales, w_bit=4, group_size=128, bias
     if x.shape[0] == 0:
         return torch.zeros(out_shape, dtype=x.dtype, device=x.device)
     tokens = x.numel() // x.shape[-1]
-    if USE_DEQUANT_MATMUL and tokens >= dequant_matmul_token_threshold(x.shape[-1]):
-        w = awq_dequantize_triton(qweight, scales, qzeros)
-        out = torch.matmul(x, w.to(x.dtype))
-        out = out + bias if bias is not None else out
+    if USE_DEQUANT_MATMUL and tokens >= dequant_matmul_token_threshold(x.shape[-1], out_features):
+        if group_size % 8 == 0 and x.dtype == torch.float16:
+            # dequantize (transposed, fp16 [N, K]) + this package's own fp16 MFMA GEMM: no vendor library on the path
+            out = gemm_f16(x.reshape(-1, x.shape[-1]), awq_dequantize_transposed(qweight, scales, qzeros), bias)
+        else:
+            w = awq_dequantize_triton(qweight, scales, qzeros)
+            out = torch.matmul(x, w.to(x.dtype))
+            out = out + bias if bias is not None else out
     else:
         out = awq_gemm_triton(x.reshape(-1, x.shape[-1]), qweight, scales, qzeros, split_k_iters=8, bias=bias)
     out = out.reshape(out_shape)

@@ -122,7 +122,7 @@ def test_module_paths_agree_around_the_token_threshold(cuda, K):
     qw, qz, sc = W.awq_weights(N, K, 4242)
     m = WQLinear_GEMM(4, 128, K, N, False, cuda)
     m.qweight, m.qzeros, m.scales = qw.to(cuda), qz.to(cuda), sc.to(cuda)
-    t = dequant_matmul_token_threshold(K)
+    t = dequant_matmul_token_threshold(K, N)
     assert t < 1024
     for M in (t - 1, t):
         x = W.activations(M, K, 4300 + M, dtype=torch.float16, outliers=False)
@@ -254,3 +254,61 @@ def test_decode_kernel_extreme_nibbles_and_zero_tokens(cuda, force_awq_plan):
             force_awq_plan(variant, 0)
             out = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8)
             assert rel_err(out, ref) <= REL_TOL, (qv, zv, variant)
+
+
+@pytest.mark.parametrize("K,N,G", [(3584, 4608, 128), (896, 4864, 128), (256, 264, 64), (128, 8, 32), (512, 1000, 512),
+                                   (8, 520, 8), (72, 40, 72)])
+def test_dequant_transposed_bit_exact(cuda, K, N, G):
+    """The transposed dequantizer (fp16 [N, K], the GEMM's weight operand): the oracle's dequantized matrix, transposed,
+    bit for bit; K that is not a multiple of its 64-row tiles, N / 8 that is not a multiple of its 32-word tiles."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_dequantize_transposed
+    qw, qz, s = W.awq_weights(N, K, K + N, group=G)
+    ref = R.awq_dequantize(qw, qz, s, G)
+    out = awq_dequantize_transposed(qw.to(cuda), s.to(cuda), qz.to(cuda))
+    assert out.dtype == torch.float16 and out.shape == (N, K)
+    assert torch.equal(out.cpu().view(torch.int16), ref.t().contiguous().view(torch.int16))
+
+
+@pytest.mark.parametrize("M,K,N", [(1024, 3584, 4608), (300, 520, 1000), (65, 72, 40), (2048, 1024, 512), (1, 128, 8)])
+def test_gemm_f16_against_fp64(cuda, M, K, N):
+    """The fp16 MFMA GEMM (fp32 accumulation): raw accumulators against an fp64 product of the same fp16 operands, the
+    fp16 output with and without bias; ragged M / N, K that is not a multiple of the K tile."""
+    from llmqrt_amd.awq_kernels import gemm_f16
+    g = torch.Generator().manual_seed(M + K + N)
+    x = torch.randn(M, K, generator=g).half()
+    w = (torch.randn(N, K, generator=g) * 0.05).half()
+    bias = torch.randn(N, generator=g).half()
+    ref = x.double() @ w.double().t()
+    dump = torch.empty((M, N), dtype=torch.float32, device=cuda)
+    y = gemm_f16(x.to(cuda), w.to(cuda), _acc_dump=dump)
+    assert rel_err(dump, ref) <= 1e-5
+    assert rel_err(y, ref) <= 1e-3
+    yb = gemm_f16(x.to(cuda), w.to(cuda), bias.to(cuda))
+    assert rel_err(yb, ref + bias.double()) <= 1e-3
+
+
+def test_module_many_token_path_is_own_kernels(cuda):
+    """Above its token threshold WQLinear_GEMM runs the transposed dequantizer and the fp16 MFMA GEMM of this library
+    (no torch.matmul): output within tolerance of the oracle, with bias, 3-D input."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.linear import WQLinear_GEMM
+    from llmqrt_amd.linear.linear_awq import dequant_matmul_token_threshold
+    K, N = 1024, 1056
+    qw, qz, s = W.awq_weights(N, K, 77)
+    mod = WQLinear_GEMM(4, 128, K, N, True, cuda)
+    mod.qweight.copy_(qw); mod.qzeros.copy_(qz); mod.scales.copy_(s)
+    mod.bias.copy_((0.1 * torch.randn(N, generator=torch.Generator().manual_seed(3))).half())
+    T = dequant_matmul_token_threshold(K, N) + 64
+    x = W.activations(T, K, 78, dtype=torch.float16, outliers=False)
+    ref = (R.awq_gemm(x, qw, qz, s, 128).float() + mod.bias.float().cpu()).half()
+    real_matmul = torch.matmul
+    try:
+        def no_matmul(*a, **k):
+            raise AssertionError("torch.matmul must not run on this path")
+        torch.matmul = no_matmul
+        y = mod(x.to(cuda).view(2, T // 2, K))
+    finally:
+        torch.matmul = real_matmul
+    assert y.shape == (2, T // 2, N)
+    assert rel_err(y.reshape(T, N), ref) <= REL_TOL
