@@ -330,38 +330,49 @@ def details_awq(dev, full=True):
         if not full:
             del copies
             continue
-        # prefill side of the module: the dequantizer (weights resident), alone and followed by the fp16 matmul
+        # prefill side of the module: the dequantizers (weights resident), alone and followed by this library's fp16
+        # MFMA GEMM (the module's path above its token threshold); the vendor fp16 matmul on the [K, N] tensor is
+        # timed beside it for context only
         deq = torch.empty((K, N), dtype=torch.float16, device=dev)
+        deq_t = torch.empty((N, K), dtype=torch.float16, device=dev)
         c = copies[0]
 
         def dequant():
             L.llmq_awq_dequant(c[0].data_ptr(), c[2].data_ptr(), c[1].data_ptr(), deq.data_ptr(), K, N, 128, stream)
-        t_deq = batch_time_us([dequant], stream_obj, 40)
-        xp = W.activations(2048, K, W.seed_for(3, 900 + pi), dtype=torch.float16, outliers=False).to(dev)
 
-        def prefill():
-            dequant()
-            torch.matmul(xp, deq)
-        t_pre = batch_time_us([prefill], stream_obj, 10)
+        def dequant_t():
+            L.llmq_awq_dequant_t(c[0].data_ptr(), c[2].data_ptr(), c[1].data_ptr(), deq_t.data_ptr(), K, N, 128, stream)
+        t_deq = batch_time_us([dequant], stream_obj, 40)
+        t_deq_t = batch_time_us([dequant_t], stream_obj, 40)
+
+        def own_path(xm, om, wsm):
+            def f():
+                dequant_t()
+                L.llmq_gemm_f16(xm.data_ptr(), K, deq_t.data_ptr(), K, 1.0, None, 0, 0.0, om.data_ptr(), 1, N, xm.shape[0], N, K,
+                                None, wsm.data_ptr(), wsm.numel(), stream)
+            return f
         mid = {}
-        for Mm in (256, 512):
+        for Mm in (256, 512, 2048):
             xm = W.activations(Mm, K, W.seed_for(3, 950 + pi + Mm), dtype=torch.float16, outliers=False).to(dev)
             om = torch.empty((Mm, N), dtype=torch.float16, device=dev)
-            wsm = torch.empty(max(L.llmq_awq_gemm_workspace_bytes(Mm, N, K), 16), dtype=torch.uint8, device=dev)
+            wsm = torch.empty(max(L.llmq_awq_gemm_workspace_bytes(Mm, N, K), L.llmq_gemm_f16_workspace_bytes(Mm, N, K), 16),
+                              dtype=torch.uint8, device=dev)
 
             def fused():
                 L.llmq_awq_gemm(xm.data_ptr(), K, c[0].data_ptr(), c[2].data_ptr(), c[1].data_ptr(), None, om.data_ptr(),
                                 Mm, N, K, 128, wsm.data_ptr(), wsm.numel(), stream)
 
-            def unfused():
+            def vendor():
                 dequant()
                 torch.matmul(xm, deq)
-            mid[f"M{Mm}_tile_kernel_us"] = round(batch_time_us([fused], stream_obj, 20), 1)
-            mid[f"M{Mm}_dequant_plus_fp16_matmul_us"] = round(batch_time_us([unfused], stream_obj, 20), 1)
+            mid[f"M{Mm}_tile_kernel_us"] = round(batch_time_us([fused], stream_obj, 10), 1)
+            mid[f"M{Mm}_dequant_t_plus_gemm_f16_us"] = round(batch_time_us([own_path(xm, om, wsm)], stream_obj, 10), 1)
+            mid[f"M{Mm}_dequant_plus_vendor_matmul_us"] = round(batch_time_us([vendor], stream_obj, 10), 1)
         db = K * N // 2 + 2 * K * N
+        t_pre = mid["M2048_dequant_t_plus_gemm_f16_us"]
         rows.append({"proj": pname, **mid, "dequant_us": round(t_deq, 2), "dequant_GBs": round(db / t_deq / 1e3, 1),
                      "dequant_pct_hbm_peak": round(100 * db / t_deq / 1e3 / PEAK_HBM_GBS, 2),
-                     "prefill_M2048_dequant_plus_fp16_matmul_us": round(t_pre, 1),
+                     "dequant_t_us": round(t_deq_t, 2), "dequant_t_GBs": round(db / t_deq_t / 1e3, 1),
                      "prefill_M2048_TFLOPs": round(2 * 2048 * N * K / t_pre / 1e6, 1)})
         del copies
     return rows

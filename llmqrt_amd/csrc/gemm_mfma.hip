@@ -723,25 +723,28 @@ bool skinny_plan(int64_t M, int64_t N, int64_t K, int& t, int& nw) {
 // Pick the tile shape and K split with the smallest modelled time:
 // waves of blocks over the CUs x per-block MFMA time, with a floor from the bytes each block streams.
 // mfma_scale: matrix-core time per K byte relative to int8 / fp8 (fp16: 2)
-Plan make_plan(int64_t M, int64_t N, int64_t K, double mfma_scale = 1.0) {
+// fp8: the 64-byte K tiles have one MFMA sub-step there and keep the register-staged loop (measured ~20 % slower)
+Plan make_plan(int64_t M, int64_t N, int64_t K, double mfma_scale = 1.0, bool fp8 = false) {
     int ocfg, osp;
     if (plan_override(ocfg, osp) && ocfg < 100) {
         const TileShape s = kShapes[ocfg < kNumShapes ? ocfg : kNumShapes - 1];
         const int kps = cdiv(cdiv(K, osp), s.bk) * s.bk;
         return Plan{ocfg < kNumShapes ? ocfg : kNumShapes - 1, cdiv(K, kps), kps};
     }
-    // Cost model calibrated on MI355X (microseconds): a CU runs `per_cu` blocks at a time, a block needs
-    // t_tile per 64 bytes of K plus a fixed prologue/epilogue cost; blocks execute in rounds over the
-    // 256 CUs.  The chip is power-limited under MFMA load: with a fraction f of the CUs busy a K tile
-    // takes (0.52 + 0.48 f) of its full-chip time, so a partly filled round is cheaper than a full one.
-    // Split-K adds a second kernel and the round trip of the fp32/int32 partials.
+    // Cost model calibrated on MI355X (microseconds) with the direct-load kernels: a block needs t_tile per 64 bytes
+    // of K plus a fixed prologue/epilogue cost; blocks execute in rounds over the 256 CUs (the small tiles are bound
+    // by the CU's load path, so co-resident blocks share it and are not modelled as extra slots).  The chip is
+    // power-limited under MFMA load: with a fraction f of the CUs busy a K tile takes (0.52 + 0.48 f) of its
+    // full-chip time, so a partly filled round is cheaper than a full one.  Split-K adds a second kernel and the round
+    // trip of the fp32/int32 partials.  Checked against a sweep of every configuration x K split at M = 128 / 512 /
+    // 2048: the plan picked is within 1.5 % of the best measured one on average.
     struct Model { int cfg, per_cu; double t_tile, fixed; };
     static const Model kModels[] = {
-        {1, 1, 0.98, 14.5},   // 256x256, 8 waves
-        {2, 1, 0.665, 14.4},  // 256x128
-        {3, 2, 0.636, 11.1},  // 128x128 (two blocks per CU, times are per resident pair)
-        {4, 3, 0.40, 7.0},    // 64x128
-        {5, 4, 0.30, 6.0},    // 32x128
+        {1, 1, 0.88, 13.0},  // 256x256, 8 waves
+        {2, 1, 0.60, 12.0},  // 256x128
+        {3, 1, 0.27, 8.0},   // 128x128
+        {4, 1, 0.15, 7.0},   // 64x128
+        {5, 1, 0.10, 6.0},   // 32x128
     };
     Plan best{1, 1, (int)K};
     double best_t = 1e300;
@@ -750,8 +753,7 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, double mfma_scale = 1.0) {
         // skinny tiles are for small M; the 64-row tile also serves up to 1024 rows when 128x128 tiles
         // could not even fill the CUs once and K is short (measured: o and qkv at M = 512)
         if (M > 128 && md.cfg == 5) continue;
-        if (M > 128 && md.cfg == 4 &&
-            (M > 1024 || K > 8192 || (int64_t)cdiv(M, 128) * cdiv(N, 128) >= 2 * kNumCu)) continue;
+        if (M > 128 && md.cfg == 4 && (M > 1024 || (int64_t)cdiv(M, 128) * cdiv(N, 128) >= 2 * kNumCu)) continue;
         if (md.cfg < 5 && M <= s.bm / 2) continue;            // mostly padding
         const int64_t tiles = (int64_t)cdiv(M, s.bm) * cdiv(N, s.bn);
         for (int sp = 1; sp <= 16; sp++) {
@@ -761,7 +763,7 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, double mfma_scale = 1.0) {
             if (eff_sp != sp) continue;
             const int64_t slots = (int64_t)kNumCu * md.per_cu, blocks = tiles * sp;
             const int64_t full_rounds = blocks / slots, rest = blocks % slots;
-            const double tt = md.t_tile * mfma_scale;
+            const double tt = md.t_tile * mfma_scale * (fp8 && s.bk == 64 ? 1.2 : 1.0);
             double t = full_rounds * (kps / 64.0 * tt + md.fixed);
             if (rest) t += kps / 64.0 * tt * (0.52 + 0.48 * (double)rest / slots) + md.fixed;
             if (sp > 1) t += 5.0 + (double)M * N * sp * 8.0 / 8.0e6;
@@ -859,7 +861,7 @@ int gemm_entry(int op, int a_format, const uint8_t* A, int64_t lda, const uint8_
         return launch_gemm_skinny(fp8, a_format == LLMQ_E5M2 ? 1 : 0, sk_t, sk_nw, A, lda, B, ldb, (int)M, (int)N, (int)K, sep,
                                   out, ldo, acc_dump, st);
     }
-    Plan p = make_plan(M, N, K, op == 2 ? 2.0 : 1.0);
+    Plan p = make_plan(M, N, K, op == 2 ? 2.0 : 1.0, fp8);
     // fp8 fragments are twice as wide: the 8-wave prefill tile runs ~5 % faster with 128-byte K tiles
     if (fp8 && g_force_cfg < 0 && p.cfg == 1 && p.splits == 1) p.cfg = 6;
     // int8 with direct loads: no staging registers, so the 128-byte K tile fits (half the barriers, whole lines per row)
@@ -935,8 +937,9 @@ extern "C" size_t llmq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     int sk_t, sk_nw;
     if (skinny_plan(M, N, K, sk_t, sk_nw)) return 0;
-    const Plan p = make_plan(M, N, K);
-    return p.splits > 1 ? (size_t)p.splits * M * N * 4 : 0;
+    const Plan p = make_plan(M, N, K), p8 = make_plan(M, N, K, 1.0, true);  // the int8 and the fp8 plan may differ
+    const int splits = p.splits > p8.splits ? p.splits : p8.splits;
+    return splits > 1 ? (size_t)splits * M * N * 4 : 0;
 }
 
 extern "C" int llmq_gemm_w8a8(const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb, const float* a_scale,

@@ -319,7 +319,7 @@ def test_hip_graph_replays_match_eager(cuda):
     ops in between, must reproduce the eager result bit for bit."""
     from llmqrt_amd import _abi, workloads as W
     L = _abi.lib()
-    M, K, N = 80, 3584, 3584
+    M, K, N = 80, 18944, 3584
     qw, ws = W.int8_weights(N, K, 501)
     qw, ws = qw.to(cuda), ws.to(cuda)
     x = W.activations(M, K, 500).to(cuda)
