@@ -34,11 +34,11 @@ if ROOT not in sys.path:
 # WRITE_SIZE of two `rocprofv3 --pmc` runs of `bench.py --roofline-only`, each scaled by what the same
 # counter reads for the 256 MiB calibration copy (2.000 and 1.000); see
 # profiles/gemm_w8a8_int8_mfma_prefill_qwen2_7b.md.  A measured constant: counters cannot be read from here.
-ROOFLINE_TRAFFIC_BYTES = 628724706
+ROOFLINE_TRAFFIC_BYTES = 634612253
 # The same for the FP8 launches (bench.py --fp8-only, profiles/gemm_fp8_mfma_prefill_qwen2_7b.md) and the W4A16
 # decode launches at M <= 16 (bench.py --awq-only, profiles/awq_gemv_w4a16_decode_qwen2_7b.md); None = not measured.
-FP8_TRAFFIC_BYTES = None
-W4A16_TRAFFIC_BYTES = None
+FP8_TRAFFIC_BYTES = 299021694
+W4A16_TRAFFIC_BYTES = 34500000
 CPU_BASELINE_REPS = 12        # bounded CPU sample: about 10-15 s of host work
 PEAK_INT8_TOPS = 5033.0   # dense int8 MFMA peak of MI355X, TOP/s (256 CU x 2.4 GHz x 8192 op/clk)
 PEAK_FP8_TFLOPS = 5033.0  # dense fp8 MFMA peak
@@ -64,6 +64,9 @@ def parse_args():
     ap.add_argument("--fp8-only", action="store_true",
                     help="profiler mode: only the FP8 GEMM launches (4 projections x M in {512, 4096}), preceded by "
                          "one 256 MiB calibration copy")
+    ap.add_argument("--micro", action="store_true",
+                    help="hardware microbenchmarks instead of the workload: register-only MFMA rate (random / zero "
+                         "operands), LDS bandwidth per CU, and HBM streaming rate of a packed W4 matrix by access pattern")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant kernel's launches (for rocprofv3 summaries)")
     return ap.parse_args()
@@ -564,6 +567,35 @@ def details_norm_quant(dev):
     return out
 
 
+def micro():
+    """Microbenchmarks of the resources that bound the kernels (llmqrt_amd/csrc/microbench.hip); one JSON line."""
+    import ctypes
+    path = os.path.join(ROOT, "llmqrt_amd", "lib", "libllmq_microbench_gfx950.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: run `python -m llmqrt_amd.csrc.build`")
+    mb = ctypes.CDLL(path)
+    val = ctypes.c_double()
+
+    def call(fn, *a):
+        rc = fn(*[ctypes.c_int(v) for v in a], ctypes.byref(val))
+        if rc != 0:
+            raise RuntimeError(f"{fn.__name__}{a} failed with {rc}")
+        return val.value
+
+    out = {"micro": True, "mfma_TOPS": {}, "lds_bytes_per_ns_per_cu": {}, "w4_stream_GBs": {}}
+    for kind, name in enumerate(("int8_32x32x32", "fp8_32x32x64", "fp16_32x32x16")):
+        for data, dn in enumerate(("random", "zero")):
+            out["mfma_TOPS"][f"{name}_{dn}"] = round(call(mb.llmq_mb_mfma, kind, data), 1)
+    for mode, name in enumerate(("ds_read_b128", "ds_write_b128", "global_load_lds_dwordx4")):
+        out["lds_bytes_per_ns_per_cu"][name] = round(call(mb.llmq_mb_lds, mode), 1)
+    # packed AWQ weights of the Qwen2-7B projections, [K, N/8] int32; rows_per_wave = K / (waves x K splits)
+    for pname, K, N in (("qkv", 3584, 4608), ("gate_up", 3584, 37888), ("down", 18944, 3584)):
+        for mode, mn in enumerate(("regs", "regs_lds_roundtrip", "load_to_lds")):
+            for nw, rows in ((2, 64), (2, 128), (4, 128), (4, 448)):
+                out["w4_stream_GBs"][f"{pname}_{mn}_{nw}w_{rows}rows"] = round(call(mb.llmq_mb_stream, mode, nw, rows, K, N), 0)
+    print(json.dumps(out))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -580,6 +612,9 @@ def main():
     stream_obj = torch.cuda.current_stream()
     stream = stream_obj.cuda_stream
 
+    if args.micro:
+        micro()
+        return
     if args.awq_only:
         awq_only(dev, args.steps, args.warmup)
         return

@@ -266,7 +266,7 @@ __global__ __launch_bounds__(C::NT) void awq_tile_kernel(
                 }
                 const int n = nb + 16 * g + 8 * khalf;  // 8 consecutive channels; N % 8 == 0: all in or all out
                 if (m_ok && n < N)
-                    *reinterpret_cast<uint4*>(orow + n) = make_uint4(pk[2 * g][0], pk[2 * g][1], pk[2 * g + 1][0], pk[2 * g + 1][1]);
+                    store_streaming(orow + n, make_uint4(pk[2 * g][0], pk[2 * g][1], pk[2 * g + 1][0], pk[2 * g + 1][1]));
             }
         }
     }

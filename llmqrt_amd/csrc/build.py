@@ -15,6 +15,7 @@ ROOT = HERE.parent.parent
 OUT_DIR = HERE.parent / "lib"
 OBJ_DIR = OUT_DIR / "obj"
 LIB = OUT_DIR / "libllmq_gfx950.so"
+MICROBENCH_LIB = OUT_DIR / "libllmq_microbench_gfx950.so"  # hardware microbenchmarks for `bench.py --micro`; not the product
 SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "gemm_skinny.hip", "awq.hip", "awq_decode.hip", "awq_tile.hip"]
 
 HIPCC_FLAGS = [
@@ -22,6 +23,7 @@ HIPCC_FLAGS = [
     # packed-fp32 VALU ops are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-Wno-inline-asm",  # the LDS-DMA asm names m0 as clobbered on purpose
     f"-I{ROOT / 'include'}", f"-I{HERE}",
 ]
 
@@ -38,16 +40,21 @@ def _compile(src: str) -> pathlib.Path:
     return obj
 
 
-def build(verbose: bool = True) -> pathlib.Path:
-    OBJ_DIR.mkdir(parents=True, exist_ok=True)
-    with concurrent.futures.ThreadPoolExecutor(max_workers=4) as ex:
-        objs = list(ex.map(_compile, SOURCES))
-    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *map(str, objs)]
+def _link(lib: pathlib.Path, objs) -> None:
+    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(lib), *map(str, objs)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+
+
+def build(verbose: bool = True) -> pathlib.Path:
+    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=4) as ex:
+        objs = list(ex.map(_compile, SOURCES + ["microbench.hip"]))
+    _link(LIB, objs[:-1])
+    _link(MICROBENCH_LIB, objs[-1:])
     if verbose:
-        print(f"built {LIB}")
+        print(f"built {LIB}\nbuilt {MICROBENCH_LIB}")
     return LIB
 
 

@@ -499,7 +499,7 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
                     for (int it = 0; it < 8; it++) {
                         const int q = it * kWave + lane, row = q >> 3, c = q & 7;
                         const uint4 v = region[row * 8 + (c ^ ((row >> 1) & 7))];
-                        *reinterpret_cast<uint4*>(obase + (int64_t)row * ldo + 8 * c) = v;
+                        store_streaming(obase + (int64_t)row * ldo + 8 * c, v);
                     }
                 }
                 return;
@@ -546,8 +546,7 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
                             pk[2 * g][x] = sw2[0];
                             pk[2 * g + 1][x] = sw2[1];
                         }
-                        *reinterpret_cast<uint4*>(orow + nb + 16 * g + 8 * khalf) =
-                            make_uint4(pk[2 * g][0], pk[2 * g][1], pk[2 * g + 1][0], pk[2 * g + 1][1]);
+                        store_streaming(orow + nb + 16 * g + 8 * khalf, make_uint4(pk[2 * g][0], pk[2 * g][1], pk[2 * g + 1][0], pk[2 * g + 1][1]));
                     }
                 }
             }
@@ -766,6 +765,9 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, double mfma_scale = 1.0, bool fp
             const double tt = md.t_tile * mfma_scale * (fp8 && s.bk == 64 ? 1.2 : 1.0);
             double t = full_rounds * (kps / 64.0 * tt + md.fixed);
             if (rest) t += kps / 64.0 * tt * (0.52 + 0.48 * (double)rest / slots) + md.fixed;
+            // two 64-row blocks fit a CU side by side and share its load path: between one and two blocks per CU the
+            // launch is one stretched round, not two (measured: 288 blocks of K = 3584 take 20 us, 224 take 14)
+            if (md.cfg == 4 && blocks > slots && blocks <= 2 * slots) t = kps / 64.0 * tt * blocks / slots + md.fixed + 3.0;
             if (sp > 1) t += 5.0 + (double)M * N * sp * 8.0 / 8.0e6;
             if (t < best_t) { best_t = t; best = Plan{md.cfg, sp, kps}; }
         }

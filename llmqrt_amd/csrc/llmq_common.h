@@ -25,6 +25,13 @@ template <> struct Lo<LLMQ_F16> {
     static __device__ __forceinline__ float round(float f) { return to_f32(from_f32(f)); }
 };
 
+// 16-byte store of finished output with the non-temporal hint: the tile is not read again by this kernel, and
+// without the hint its lines are allocated in L2 beside the operand panels the other tiles of the XCD still need
+// (measured on 8192 x 37888 x 3584: 1177 -> 1042 us, the same as storing into a cache-resident dummy region).
+__device__ __forceinline__ void store_streaming(void* p, uint4 v) {
+    typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+    __builtin_nontemporal_store(u4v{v.x, v.y, v.z, v.w}, reinterpret_cast<u4v*>(p));
+}
 __device__ __forceinline__ float load_as_f32(const void* p, int dtype, int64_t i) {
     if (dtype == LLMQ_F32) return ((const float*)p)[i];
     uint16_t h = ((const uint16_t*)p)[i];

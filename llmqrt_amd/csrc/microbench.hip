@@ -1,0 +1,283 @@
+// Microbenchmarks of the MI355X resources that bound the kernels of this library (built into a library of their
+// own, libllmq_microbench_gfx950.so, and run by `bench.py --micro`; no part of the product path):
+//   llmq_mb_mfma    matrix-core throughput of a register-only MFMA loop (int8 32x32x32 / fp8 32x32x64 / fp16
+//                   32x32x16), operands random or all zero: what the chip sustains under its power management
+//                   with no memory traffic at all;
+//   llmq_mb_lds     LDS bandwidth per CU of ds_read_b128, ds_write_b128 and global_load_lds_dwordx4;
+//   llmq_mb_stream  how fast the packed AWQ weight matrix [K, N/8] int32 streams out of HBM as a function of the
+//                   access pattern (128-byte row segments, eight 16-byte loads per lane): short-lived wavefronts
+//                   that request their whole share at once against wavefronts that loop, with the data consumed
+//                   from registers, passed through LDS (as a layout change needs), or loaded straight into LDS.
+// Each function allocates what it needs, times its kernel with HIP events and returns 0 on success.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdlib.h>
+
+#include <algorithm>
+#include <vector>
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+#define MB_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define MB_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define MB_CK(x) do { if ((x) != hipSuccess) return 1; } while (0)
+
+// ---- matrix cores: 4 x 4 independent 32x32 accumulators per wavefront, one wavefront per SIMD ------------------
+template <int KIND>
+__global__ __launch_bounds__(256) void mfma_kernel(int iters, const v4i* src, int* out) {
+    v4i a[4], b[4];
+    for (int i = 0; i < 4; i++) {
+        a[i] = src[(threadIdx.x * 8 + i) & 4095];
+        b[i] = src[(threadIdx.x * 8 + 4 + i) & 4095];
+    }
+    v16i c[4][4];
+    for (int i = 0; i < 4; i++)
+        for (int j = 0; j < 4; j++)
+            for (int r = 0; r < 16; r++) c[i][j][r] = 0;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (KIND == 0) {
+                    c[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], c[i][j], 0, 0, 0);
+                } else if (KIND == 1) {
+                    const v4i a2 = a[(i + 1) & 3], b2 = b[(j + 1) & 3];
+                    const v8i a8 = {a[i][0], a[i][1], a[i][2], a[i][3], a2[0], a2[1], a2[2], a2[3]};
+                    const v8i b8 = {b[j][0], b[j][1], b[j][2], b[j][3], b2[0], b2[1], b2[2], b2[3]};
+                    c[i][j] = (v16i)__builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, (v16f)c[i][j], 0, 0, 0, 0, 0, 0);
+                } else {
+                    c[i][j] = (v16i)__builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a[i]), __builtin_bit_cast(v8h, b[j]),
+                                                                           (v16f)c[i][j], 0, 0, 0);
+                }
+            }
+    }
+    int s = 0;
+    for (int i = 0; i < 4; i++)
+        for (int j = 0; j < 4; j++)
+            for (int r = 0; r < 16; r++) s += c[i][j][r];
+    if (s == 123456789) out[0] = s;
+}
+
+// ---- LDS: every wavefront moves 8 KB per iteration, 1 KB per instruction ---------------------------------------
+template <int MODE>
+__global__ __launch_bounds__(512) void lds_kernel(const uint4* __restrict__ src, uint32_t* out, int iters) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid & 63;
+    uint4 v = src[tid];
+    uint32_t acc = 0;
+    const uint32_t la = (uint32_t)(uintptr_t)MB_LPTR(smem + wave * 8192 + lane * 16);
+    if (MODE == 0) {
+        for (int i = 0; i < iters; i++) {
+            u4 r[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r[j]) : "v"(la), "n"(j * 1024) : "memory");
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc += r[j].x;
+        }
+    } else if (MODE == 1) {
+        const u4 vv = {v.x, v.y, v.z, v.w};
+        for (int i = 0; i < iters; i++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(la), "v"(vv), "n"(j * 1024) : "memory");
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+    } else {
+        const uint8_t* g = reinterpret_cast<const uint8_t*>(src) + (size_t)blockIdx.x * 8192 + wave * 1024;  // cache-resident source
+        for (int i = 0; i < iters; i++) {
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                __builtin_amdgcn_global_load_lds(MB_GPTR(g + lane * 16 + (j & 1) * 512), MB_LPTR(smem + wave * 8192 + j * 1024), 16, 0, 0);
+            asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    out[blockIdx.x * 512 + tid] = acc + reinterpret_cast<uint32_t*>(smem)[tid] + v.x;
+}
+
+// ---- HBM streaming of the packed weight matrix: 128-byte segments, 8 rows per instruction, 8 loads per pass -----
+template <int MODE, int NW>
+__global__ __launch_bounds__(NW * 64) void stream_kernel(const u4* __restrict__ w, int K, int Nq, int tiles_n, int rows_per_wave,
+                                                         uint32_t* out) {
+    __shared__ __attribute__((aligned(16))) uint8_t smem[NW * (MODE == 2 ? 16384 : 8192)];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tile = blockIdx.x % tiles_n, ks = blockIdx.x / tiles_n;
+    const int col = min(tile * 8 + (lane & 7), Nq - 1);
+    const int k0 = min(K, (ks * NW + wave) * rows_per_wave), k1 = min(K, k0 + rows_per_wave);
+    const int npass = (k1 - k0) / 64;  // a pass = 64 rows x 128 bytes = 8 KB
+    uint32_t acc = 0;
+    const u4* base = w + (int64_t)(k0 + (lane >> 3)) * Nq + col;
+    uint8_t* ring = smem + wave * (MODE == 2 ? 16384 : 8192);
+    if (npass > 0) {
+        if (MODE == 2) {
+            auto issue = [&](int p, int slot) {
+                const u4* b = base + (int64_t)min(p, npass - 1) * 64 * Nq;
+#pragma unroll
+                for (int u = 0; u < 8; u++)
+                    __builtin_amdgcn_global_load_lds(MB_GPTR(b + (int64_t)u * 8 * Nq), MB_LPTR(ring + slot * 8192 + u * 1024), 16, 0, 0);
+            };
+            issue(0, 0);
+            for (int p = 0; p < npass; p++) {
+                issue(p + 1, (p + 1) & 1);
+                asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                uint32_t t;
+                const uint32_t a = (uint32_t)(uintptr_t)MB_LPTR(ring + (p & 1) * 8192) + lane * 4;
+                asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(t) : "v"(a) : "memory");
+                acc ^= t;
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        } else {
+            u4 v[8];
+            auto issue = [&](int p) {
+                const u4* b = base + (int64_t)min(p, npass - 1) * 64 * Nq;
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = b[(int64_t)u * 8 * Nq];
+            };
+            issue(0);
+            for (int p = 0; p < npass; p++) {
+                if (MODE == 1) {
+#pragma unroll
+                    for (int u = 0; u < 8; u++) *reinterpret_cast<u4*>(ring + u * 1024 + lane * 16) = v[u];
+                    issue(p + 1);
+                    const uint32_t* l = reinterpret_cast<const uint32_t*>(ring);  // read back as a matrix-core operand layout would
+#pragma unroll
+                    for (int c = 0; c < 2; c++)
+#pragma unroll
+                        for (int s = 0; s < 2; s++)
+#pragma unroll
+                            for (int r = 0; r < 8; r++) acc ^= l[(c * 32 + 8 * (lane >> 4) + r) * 32 + 16 * s + (lane & 15)];
+                } else {
+                    uint32_t t = 0;
+#pragma unroll
+                    for (int u = 0; u < 8; u++) t ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+                    acc ^= t;
+                    issue(p + 1);
+                }
+            }
+        }
+    }
+    if (acc == 0x12345679u) out[0] = acc;
+}
+
+template <class F>
+int time_ms(F launch, int reps, float* ms) {
+    hipEvent_t e0, e1;
+    MB_CK(hipEventCreate(&e0));
+    MB_CK(hipEventCreate(&e1));
+    launch();
+    MB_CK(hipDeviceSynchronize());
+    float best = 1e30f;
+    for (int rep = 0; rep < 3; rep++) {
+        MB_CK(hipEventRecord(e0));
+        for (int i = 0; i < reps; i++) launch();
+        MB_CK(hipEventRecord(e1));
+        MB_CK(hipEventSynchronize(e1));
+        float t;
+        MB_CK(hipEventElapsedTime(&t, e0, e1));
+        best = std::min(best, t / reps);
+    }
+    MB_CK(hipEventDestroy(e0));
+    MB_CK(hipEventDestroy(e1));
+    *ms = best;
+    return 0;
+}
+
+}  // namespace
+
+// kind: 0 int8 32x32x32, 1 fp8 32x32x64, 2 fp16 32x32x16.  data: 0 random bytes, 1 all zero.  -> TOP/s (TFLOP/s)
+extern "C" int llmq_mb_mfma(int kind, int data, double* tops) {
+    std::vector<unsigned char> h(65536, 0);
+    srand(1);
+    if (data == 0)
+        for (size_t i = 0; i < h.size(); i += 2) {
+            unsigned char lo = rand() & 0xff, hi = rand() & 0xff;
+            if (kind == 1) {  // e4m3: every byte random, the two NaN encodings excepted
+                if ((lo & 0x7f) == 0x7f) lo ^= 1;
+                if ((hi & 0x7f) == 0x7f) hi ^= 1;
+            } else if (kind == 2) {  // fp16: random sign and mantissa, exponent field in 8..15 (finite, |x| < 2)
+                hi = (hi & 0x83) | (unsigned char)((8 + (rand() & 7)) << 2);
+            }
+            h[i] = lo;
+            h[i + 1] = hi;
+        }
+    v4i* src;
+    int* out;
+    MB_CK(hipMalloc(&src, 65536));
+    MB_CK(hipMalloc(&out, 4));
+    MB_CK(hipMemcpy(src, h.data(), 65536, hipMemcpyHostToDevice));
+    const int iters = 3000, blocks = 256;
+    float ms;
+    int rc;
+    if (kind == 0) rc = time_ms([&] { mfma_kernel<0><<<blocks, 256>>>(iters, src, out); }, 1, &ms);
+    else if (kind == 1) rc = time_ms([&] { mfma_kernel<1><<<blocks, 256>>>(iters, src, out); }, 1, &ms);
+    else rc = time_ms([&] { mfma_kernel<2><<<blocks, 256>>>(iters, src, out); }, 1, &ms);
+    (void)hipFree(src);
+    (void)hipFree(out);
+    if (rc) return rc;
+    const double ops = 2.0 * 32 * 32 * (kind == 0 ? 32 : (kind == 1 ? 64 : 16));
+    *tops = (double)blocks * 4 * iters * 16 * ops / ms / 1e9;
+    return 0;
+}
+
+// mode: 0 ds_read_b128, 1 ds_write_b128, 2 global_load_lds_dwordx4 (source resident in cache).  -> bytes per nanosecond and CU
+extern "C" int llmq_mb_lds(int mode, double* bytes_per_ns_per_cu) {
+    uint4* src;
+    uint32_t* out;
+    MB_CK(hipMalloc(&src, 256 * 8192 + 65536));
+    MB_CK(hipMemset(src, 1, 256 * 8192 + 65536));
+    MB_CK(hipMalloc(&out, 256 * 512 * 4));
+    const int iters = 20000, blocks = 256;
+    float ms;
+    int rc;
+    if (mode == 0) rc = time_ms([&] { hipLaunchKernelGGL(lds_kernel<0>, dim3(blocks), dim3(512), 65536, 0, src, out, iters); }, 1, &ms);
+    else if (mode == 1) rc = time_ms([&] { hipLaunchKernelGGL(lds_kernel<1>, dim3(blocks), dim3(512), 65536, 0, src, out, iters); }, 1, &ms);
+    else rc = time_ms([&] { hipLaunchKernelGGL(lds_kernel<2>, dim3(blocks), dim3(512), 65536, 0, src, out, iters); }, 1, &ms);
+    (void)hipFree(src);
+    (void)hipFree(out);
+    if (rc) return rc;
+    *bytes_per_ns_per_cu = (double)iters * 8192 * 8 / (ms * 1e6);
+    return 0;
+}
+
+// mode: 0 registers only, 1 registers + LDS round trip, 2 global_load_lds.  The [K, N/8] int32 matrix is rotated through
+// more than 256 MB of copies so that the Infinity Cache cannot hold it.  -> GB/s
+extern "C" int llmq_mb_stream(int mode, int waves_per_block, int rows_per_wave, int K, int N, double* gbs) {
+    if ((waves_per_block != 2 && waves_per_block != 4) || rows_per_wave % 64 || N % 32 || K % 64) return 2;
+    const int Nq = N / 32;
+    const size_t bytes = (size_t)K * Nq * 16;
+    const int nc = (int)std::max<size_t>(2, ((size_t)320 << 20) / bytes + 1);
+    std::vector<u4*> w(nc, nullptr);
+    uint32_t* out;
+    MB_CK(hipMalloc(&out, 4));
+    for (int i = 0; i < nc; i++) {
+        MB_CK(hipMalloc(&w[i], bytes));
+        MB_CK(hipMemset(w[i], i + 1, bytes));
+    }
+    const int tiles_n = (Nq + 7) / 8;
+    const int splits = (K + rows_per_wave * waves_per_block - 1) / (rows_per_wave * waves_per_block);
+    const int blocks = tiles_n * splits;
+    int idx = 0;
+    auto launch = [&] {
+        const u4* p = w[idx++ % nc];
+#define MB_L(MODE, NW) stream_kernel<MODE, NW><<<blocks, NW * 64>>>(p, K, Nq, tiles_n, rows_per_wave, out)
+        if (mode == 0) { if (waves_per_block == 2) MB_L(0, 2); else MB_L(0, 4); }
+        else if (mode == 1) { if (waves_per_block == 2) MB_L(1, 2); else MB_L(1, 4); }
+        else { if (waves_per_block == 2) MB_L(2, 2); else MB_L(2, 4); }
+#undef MB_L
+    };
+    float ms;
+    const int rc = time_ms(launch, std::max(20, 2 * nc), &ms);
+    for (auto p : w) (void)hipFree(p);
+    (void)hipFree(out);
+    if (rc) return rc;
+    *gbs = bytes / (ms * 1e6);
+    return 0;
+}
