@@ -4,9 +4,13 @@
  * Conventions
  *  - Every pointer is a DEVICE pointer unless its comment says "host".
  *  - The caller owns every buffer (inputs, outputs, workspaces); the library allocates
- *    nothing, keeps no state between calls (llmq_gemm_force_plan, a tuning hook, is the one
- *    exception), never synchronises with the host and launches on the stream it is given
- *    (0 = the null stream).  Calls are asynchronous.
+ *    nothing, never synchronises with the host and launches on the stream it is given
+ *    (0 = the null stream).  Calls are asynchronous.  State kept between calls: the
+ *    *_force_plan tuning hooks, and a 1 MiB ring of arrival counters per GPU (a static device
+ *    array) for the K split of the few-token AWQ kernel, which ends inside one launch.  The
+ *    counters are zero between calls and every call takes fresh slots, so calls on different
+ *    streams do not share any; a captured call replays on the slots it was captured with, so
+ *    two replays of one graph must not run concurrently.
  *  - Matrices are row-major; `ld*` is the row stride in ELEMENTS.
  *  - Return value: LLMQ_OK (0) or a negative llmq_status; llmq_status_string() names it.
  *  - Paths below are relative to the reference's runtime/ directory.
@@ -185,7 +189,8 @@ size_t llmq_gemm_f16_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /* Tuning / test hook with no counterpart in the reference: force tile configuration `cfg`
  * (0 .. llmq_gemm_num_configs()-1) and K split `splits` for every later GEMM call of this
- * process; cfg < 0 restores the built-in heuristic.  Process-global, not thread-safe. */
+ * process; cfg < 0 restores the built-in heuristic.  cfg | 64 keeps the register-staged main loop,
+ * 100 .. 105 pick a variant of the few-token kernel.  Process-global, not thread-safe. */
 int llmq_gemm_force_plan(int cfg, int splits);
 int llmq_gemm_num_configs(void);
 

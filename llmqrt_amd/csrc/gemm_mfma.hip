@@ -63,9 +63,6 @@ struct Epilogue {
     int bias_dtype, out_dtype;
 };
 
-__device__ __forceinline__ float epi_value(float acc, float sa, float sw, float alpha, float bb) {
-    return fmaf(alpha, (acc * sa) * sw, bb);
-}
 __device__ __forceinline__ uint16_t to_out(float v, int out_dtype) {
     return out_dtype == LLMQ_BF16 ? Lo<LLMQ_BF16>::from_f32(v) : Lo<LLMQ_F16>::from_f32(v);
 }
@@ -441,33 +438,37 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
             // that a store instruction writes 8 whole 128-byte rows instead of 32 pieces of 32 bytes.
             constexpr bool LDS_EPI = LLMQ_LDS_EPILOGUE && C::TM % 2 == 0 && C::TN == 2 && C::LDS_BYTES >= (C::NT / kWave) * 8192u;
             if constexpr (LDS_EPI) {
+                // Every scale and bias value is fetched before the first output store is issued: loads and stores
+                // share one wait counter, so a load issued after a store can only be waited for together with that
+                // store's completion (microseconds when every CU writes at once).
+                float sa_r[C::TM], sw_r[2][16], bb_r[2][16];
+#pragma unroll
+                for (int i = 0; i < C::TM; i++) sa_r[i] = ep.a_scale ? ep.a_scale[m0 + wm * C::WTM + i * 32 + l32] : 1.f;
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const int n = n0 + wn * C::WTN + j * 32 + 8 * g + 4 * khalf;
+                        if (ep.w_scale) {
+                            const float4 v = *reinterpret_cast<const float4*>(ep.w_scale + n);
+                            sw_r[j][4 * g] = v.x, sw_r[j][4 * g + 1] = v.y, sw_r[j][4 * g + 2] = v.z, sw_r[j][4 * g + 3] = v.w;
+                        } else {
+                            sw_r[j][4 * g] = sw_r[j][4 * g + 1] = sw_r[j][4 * g + 2] = sw_r[j][4 * g + 3] = 1.f;
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            bb_r[j][4 * g + e] = ep.bias ? ep.beta * load_as_f32(ep.bias, ep.bias_dtype, n + e) : 0.f;
+                    }
                 __syncthreads();  // every wavefront is done reading the operand stages
                 uint4* region = lds + wave * 512;
 #pragma unroll
                 for (int p = 0; p < C::TM / 2; p++) {
 #pragma unroll
                     for (int j = 0; j < 2; j++) {
-                        // scales and bias of this 32-channel tile (re-read per pass: they sit in L1, and keeping
-                        // both tiles' worth in registers would not fit beside the accumulators)
-                        float sw[16], bb[16];
-#pragma unroll
-                        for (int g = 0; g < 4; g++) {
-                            const int n = n0 + wn * C::WTN + j * 32 + 8 * g + 4 * khalf;
-                            if (ep.w_scale) {
-                                const float4 v = *reinterpret_cast<const float4*>(ep.w_scale + n);
-                                sw[4 * g] = v.x, sw[4 * g + 1] = v.y, sw[4 * g + 2] = v.z, sw[4 * g + 3] = v.w;
-                            } else {
-                                sw[4 * g] = sw[4 * g + 1] = sw[4 * g + 2] = sw[4 * g + 3] = 1.f;
-                            }
-#pragma unroll
-                            for (int e = 0; e < 4; e++)
-                                bb[4 * g + e] = ep.bias ? ep.beta * load_as_f32(ep.bias, ep.bias_dtype, n + e) : 0.f;
-                        }
 #pragma unroll
                         for (int ii = 0; ii < 2; ii++) {
                             const int i = 2 * p + ii;
-                            const int m = m0 + wm * C::WTM + i * 32 + l32;
-                            const float sa = ep.a_scale ? ep.a_scale[m] : 1.f;
+                            const float sa = sa_r[i];
                             const int row = ii * 32 + l32, swz = (row >> 1) & 7;
                             uint32_t pk[4][2];
 #pragma unroll
@@ -476,7 +477,7 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
 #pragma unroll
                                 for (int e = 0; e < 4; e++) {
                                     const auto av = acc[i][j][4 * g + e];
-                                    h[e] = Lo<ODT>::from_f32(epi_value((float)av, sa, sw[4 * g + e], alpha, bb[4 * g + e]));
+                                    h[e] = Lo<ODT>::from_f32(epi_value((float)av, sa, sw_r[j][4 * g + e], alpha, bb_r[j][4 * g + e]));
                                 }
                                 pk[g][0] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
                                 pk[g][1] = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
@@ -504,6 +505,9 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
                 }
                 return;
             }
+            float sa_r[C::TM];  // fetched before any store is issued (see above)
+#pragma unroll
+            for (int i = 0; i < C::TM; i++) sa_r[i] = ep.a_scale ? ep.a_scale[m0 + wm * C::WTM + i * 32 + l32] : 1.f;
 #pragma unroll
             for (int j = 0; j < C::TN; j++) {
                 const int nb = n0 + wn * C::WTN + j * 32;
@@ -524,7 +528,7 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
 #pragma unroll
                 for (int i = 0; i < C::TM; i++) {
                     const int m = m0 + wm * C::WTM + i * 32 + l32;
-                    const float sa = ep.a_scale ? ep.a_scale[m] : 1.f;
+                    const float sa = sa_r[i];
                     uint32_t pk[4][2];
 #pragma unroll
                     for (int g = 0; g < 4; g++) {

@@ -151,7 +151,7 @@ __global__ __launch_bounds__(NW * kWave) void gemm_skinny_kernel(
             const int ne = min(n + e, N - 1);
             const float sw = ep.w_scale ? ep.w_scale[ne] : 1.f;
             const float bb = ep.bias ? ep.beta * load_as_f32(ep.bias, ep.bias_dtype, ne) : 0.f;
-            const float v = fmaf(alpha, ((float)sum[e] * sa) * sw, bb);
+            const float v = epi_value((float)sum[e], sa, sw, alpha, bb);
             h[e] = ep.out_dtype == LLMQ_BF16 ? Lo<LLMQ_BF16>::from_f32(v) : Lo<LLMQ_F16>::from_f32(v);
         }
         uint16_t* orow = reinterpret_cast<uint16_t*>(out) + (int64_t)m * ldo + n;

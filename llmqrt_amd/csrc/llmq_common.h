@@ -25,6 +25,16 @@ template <> struct Lo<LLMQ_F16> {
     static __device__ __forceinline__ float round(float f) { return to_f32(from_f32(f)); }
 };
 
+// GEMM epilogue value in fp32, each node rounded once: (acc * sa) * sw, then one fused multiply-add with alpha and
+// the bias term.  The result is made opaque to the compiler before it is converted to the output type: otherwise
+// the fma and a conversion to fp16 may or may not be merged into one mixed-precision instruction that rounds the
+// exact sum straight to fp16, and two code paths could disagree on ties of the double rounding.
+__device__ __forceinline__ float epi_value(float acc, float sa, float sw, float alpha, float bb) {
+    float r = fmaf(alpha, (acc * sa) * sw, bb);
+    asm volatile("" : "+v"(r));
+    return r;
+}
+
 // 16-byte store of finished output with the non-temporal hint: the tile is not read again by this kernel, and
 // without the hint its lines are allocated in L2 beside the operand panels the other tiles of the XCD still need
 // (measured on 8192 x 37888 x 3584: 1177 -> 1042 us, the same as storing into a cache-resident dummy region).

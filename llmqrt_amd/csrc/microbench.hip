@@ -8,6 +8,8 @@
 //                   access pattern (128-byte row segments, eight 16-byte loads per lane): short-lived wavefronts
 //                   that request their whole share at once against wavefronts that loop, with the data consumed
 //                   from registers, passed through LDS (as a layout change needs), or loaded straight into LDS.
+//   llmq_mb_launch  time per kernel of a chain of empty kernels on one stream, launched one by one or replayed
+//                   from a HIP graph: the floor under every short launch of the decode path.
 // Each function allocates what it needs, times its kernel with HIP events and returns 0 on success.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -279,5 +281,54 @@ extern "C" int llmq_mb_stream(int mode, int waves_per_block, int rows_per_wave, 
     (void)hipFree(out);
     if (rc) return rc;
     *gbs = bytes / (ms * 1e6);
+    return 0;
+}
+
+namespace {
+__global__ void empty_kernel(int* p) {
+    if (p && threadIdx.x == 12345) p[0] = 1;
+}
+}  // namespace
+
+// mode: 0 = n kernels launched one by one, 1 = the same n kernels captured once and replayed as a HIP graph.
+// -> microseconds per kernel (steady state, stream kept busy)
+extern "C" int llmq_mb_launch(int mode, int n, double* us_per_kernel) {
+    if (n < 1 || n > 64) return 2;
+    hipStream_t st;
+    MB_CK(hipStreamCreate(&st));
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    if (mode == 1) {
+        MB_CK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        for (int i = 0; i < n; i++) empty_kernel<<<1, 64, 0, st>>>(nullptr);
+        MB_CK(hipStreamEndCapture(st, &graph));
+        MB_CK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+    }
+    auto pass = [&] {
+        if (mode == 1) (void)hipGraphLaunch(exec, st);
+        else for (int i = 0; i < n; i++) empty_kernel<<<1, 64, 0, st>>>(nullptr);
+    };
+    hipEvent_t e0, e1;
+    MB_CK(hipEventCreate(&e0));
+    MB_CK(hipEventCreate(&e1));
+    for (int i = 0; i < 20; i++) pass();
+    MB_CK(hipStreamSynchronize(st));
+    float best = 1e30f;
+    const int reps = 200;
+    for (int rep = 0; rep < 3; rep++) {
+        MB_CK(hipEventRecord(e0, st));
+        for (int i = 0; i < reps; i++) pass();
+        MB_CK(hipEventRecord(e1, st));
+        MB_CK(hipEventSynchronize(e1));
+        float t;
+        MB_CK(hipEventElapsedTime(&t, e0, e1));
+        best = std::min(best, t);
+    }
+    *us_per_kernel = best * 1e3 / reps / n;
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipStreamDestroy(st);
     return 0;
 }

@@ -51,7 +51,7 @@ def test_argument_validation_needs_no_gpu():
     assert L.llmq_awq_gemm(p16, 100, p16, p16, p16, None, p16, 2, 64, 100, 128, None, 0, None) == -3   # K % 32
     assert L.llmq_awq_gemm(p16, 128, p16, p16, p16, None, p16, 2, 60, 128, 128, None, 0, None) == -3   # N % 8
     assert L.llmq_awq_dequant(p16, p16, p16, p16, 128, 64, 48, None) == -3                              # K % G
-    assert L.llmq_gemm_force_plan(99, 1) == -3 and L.llmq_gemm_force_plan(-1, 1) == 0
+    assert L.llmq_gemm_force_plan(99, 1) == -3 and L.llmq_gemm_force_plan(106, 1) == -3 and L.llmq_gemm_force_plan(-1, 1) == 0
     assert L.llmq_quant_workspace_bytes() >= 4096
     # split-K plans ask for a workspace, plain ones do not
     assert L.llmq_gemm_workspace_bytes(8192, 37888, 3584) == 0
