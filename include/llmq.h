@@ -187,6 +187,29 @@ int llmq_gemm_f16(const void* A, int64_t lda, const void* B, int64_t ldb, float 
                   void* workspace, size_t workspace_bytes, llmq_stream_t stream);
 size_t llmq_gemm_f16_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
+/* Few-token quantized linear in ONE launch: per-token dynamic activation quantizer + GEMM + per-token x per-channel
+ * epilogue, for M <= llmq_linear_dynamic_max_tokens(K) tokens (16, or fewer when 16 quantized rows of K + 16 bytes do not
+ * fit in 64 KB of LDS: 3 at K = 18944).  Replaces the two steps of
+ * SqW8A8BBF16OBF16PerChannel.forward / the per-token branch of FP8DynamicLinear.forward
+ * (nn_models/modules/linear/linear_sq.py:97-138 with the quantizer of lines 55-65;
+ * nn_models/modules/linear/linear_fp8.py:40-63 and 199-221) and gives, bit for bit, what
+ * llmq_quant_i8_per_token (llmq_quant_fp8_per_token) followed by llmq_gemm_w8a8 (llmq_gemm_fp8) with a_scale = the
+ * quantizer's scales, alpha = beta = 1 gives:
+ *   out[m, n] = out_dtype( ((sum_k q[m, k] B[n, k]) * s[m]) * w_scale[n] + bias[n] ).
+ * x: bf16 / f16 [M, K], row stride ldx (K % 16 == 0, ldx % 8 == 0); B: int8 / e4m3 [N, K], row stride ldb; w_scale: [N]
+ * or null; bias: [N] or null; out: bf16 / f16 [M, N].  Optional outputs for checking: q_dump [M, K] (the codes),
+ * scale_dump [M] (fp32), acc_dump [M, N] (raw accumulators).  No workspace.  More tokens return LLMQ_ERR_SHAPE. */
+int llmq_linear_i8_dynamic(const void* x, int x_dtype, int64_t ldx, const int8_t* B, int64_t ldb, const float* w_scale,
+                           const void* bias, int bias_dtype, void* out, int out_dtype, int64_t ldo, int64_t M, int64_t N,
+                           int64_t K, int8_t* q_dump, float* scale_dump, int32_t* acc_dump, llmq_stream_t stream);
+int llmq_linear_fp8_dynamic(const void* x, int x_dtype, int64_t ldx, const uint8_t* B, int64_t ldb, const float* w_scale,
+                            const void* bias, int bias_dtype, void* out, int out_dtype, int64_t ldo, int64_t M, int64_t N,
+                            int64_t K, uint8_t* q_dump, float* scale_dump, float* acc_dump, llmq_stream_t stream);
+int llmq_linear_dynamic_max_tokens(int64_t K);
+/* Tuning / test hook: 0 = two 16-channel tiles per wavefront x 4 wavefronts per block, 1 = one tile x 8 wavefronts,
+ * -1 = built-in choice.  Process-global, not thread-safe. */
+int llmq_linear_dynamic_force_variant(int v);
+
 /* Tuning / test hook with no counterpart in the reference: force tile configuration `cfg`
  * (0 .. llmq_gemm_num_configs()-1) and K split `splits` for every later GEMM call of this
  * process; cfg < 0 restores the built-in heuristic.  cfg | 64 keeps the register-staged main loop,

@@ -44,6 +44,10 @@ SIGNATURES = {
     "llmq_gemm_static_scratch_bytes": (_sz, []),
     "llmq_gemm_f16": (_int, [_vp, _i64, _vp, _i64, _f32, _vp, _int, _f32, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _sz, _vp]),
     "llmq_gemm_f16_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "llmq_linear_i8_dynamic": (_int, [_vp, _int, _i64, _vp, _i64, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "llmq_linear_fp8_dynamic": (_int, [_vp, _int, _i64, _vp, _i64, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
+    "llmq_linear_dynamic_max_tokens": (_int, [_i64]),
+    "llmq_linear_dynamic_force_variant": (_int, [_int]),
     "llmq_gemm_force_plan": (_int, [_int, _int]),
     "llmq_gemm_num_configs": (_int, []),
     "llmq_awq_gemm": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),

@@ -16,7 +16,7 @@ OUT_DIR = HERE.parent / "lib"
 OBJ_DIR = OUT_DIR / "obj"
 LIB = OUT_DIR / "libllmq_gfx950.so"
 MICROBENCH_LIB = OUT_DIR / "libllmq_microbench_gfx950.so"  # hardware microbenchmarks for `bench.py --micro`; not the product
-SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "gemm_skinny.hip", "awq.hip", "awq_decode.hip", "awq_tile.hip"]
+SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "gemm_skinny.hip", "linear_fused.hip", "awq.hip", "awq_decode.hip", "awq_tile.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -30,7 +30,9 @@ template <> struct Lo<LLMQ_F16> {
 // the fma and a conversion to fp16 may or may not be merged into one mixed-precision instruction that rounds the
 // exact sum straight to fp16, and two code paths could disagree on ties of the double rounding.
 __device__ __forceinline__ float epi_value(float acc, float sa, float sw, float alpha, float bb) {
-    float r = fmaf(alpha, (acc * sa) * sw, bb);
+    float p = (acc * sa) * sw;
+    asm volatile("" : "+v"(p));  // the scaled accumulator is a value of its own: never contracted into what follows
+    float r = fmaf(alpha, p, bb);
     asm volatile("" : "+v"(r));
     return r;
 }

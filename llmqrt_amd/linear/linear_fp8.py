@@ -10,8 +10,10 @@ from __future__ import annotations
 import torch
 
 from ..quantize import per_tensor_quantize, per_token_quantize, static_per_tensor_quantize
-from ..sq_fp8_kernels import cutlass_f8f8bf16_rowwise_sm89, cutlass_f8f8bf16_tensorwise_sm89
+from ..sq_fp8_kernels import (cutlass_f8f8bf16_rowwise_sm89, cutlass_f8f8bf16_tensorwise_sm89,
+                              dynamic_linear_max_tokens, f8f8bf16_linear_dynamic_per_token)
 from .linear_base import LinearBase
+from .linear_sq import ONE_LAUNCH_MAX_TOKENS, _fusable
 
 __all__ = ["FP8DynamicLinear", "FP8StaticLinear", "per_tensor_quantize", "per_token_quantize",
            "static_per_tensor_quantize"]
@@ -98,6 +100,12 @@ class FP8DynamicLinear(_FP8LinearBase):
             output = cutlass_f8f8bf16_tensorwise_sm89(qinput.view(-1, x_shape[-1]), qweight, self.bias, alpha, 1.0,
                                                       dtype_to_str.get(self.dtype))
         else:
+            x2 = x.reshape(-1, x_shape[-1])
+            if x2.shape[0] <= min(ONE_LAUNCH_MAX_TOKENS, dynamic_linear_max_tokens(x2.shape[-1])) and _fusable(x2):
+                # a few tokens: quantizer and GEMM in one launch (same bits as the two calls below)
+                output = f8f8bf16_linear_dynamic_per_token(x2, qweight, self.bias,
+                                                           self.weight_scale.to(torch.float32).reshape(-1).contiguous())
+                return output.view(*x_shape[:-1], -1)
             qinput, x_scale = per_token_quantize(x)
             output = cutlass_f8f8bf16_rowwise_sm89(qinput.view(-1, x_shape[-1]), qweight, self.bias,
                                                    x_scale.view(-1, 1), self.weight_scale.to(torch.float32).t(), True)

@@ -156,3 +156,55 @@ def cutlass_f8f8bf16_rowwise_sm89(XQ: torch.Tensor, WQ: torch.Tensor, bias: Opti
     _check(N <= 1 or w_scale.stride(1) == 1, f"{what}: w_scale must be contiguous")
     _check_bias(bias, WQ, N, (torch.bfloat16, torch.float32), what)
     return _run(True, XQ, WQ, x_scale, w_scale, 1.0, None, bias, 1.0, torch.bfloat16, _acc_dump)
+
+
+# ---- one-launch linears for a few tokens (no counterpart among the reference's ops: they fuse the
+# quantizer call and the GEMM op of linear_sq.py:97-138 / linear_fp8.py:199-221) ------------------------------
+
+def dynamic_linear_max_tokens(in_features: int) -> int:
+    """Largest token count the one-launch linears accept for this K (the quantized rows must fit in LDS)."""
+    return int(_abi.lib().llmq_linear_dynamic_max_tokens(int(in_features)))
+
+
+def _run_dynamic(fp8: bool, x, w, bias, w_scale, out_dtype, q_dump, scale_dump, acc_dump, what: str):
+    _check(x.dtype in (torch.bfloat16, torch.float16), f"{what}: activations must be bf16 or fp16")
+    M, N, K = _check_operands(x, w, what)
+    _check(M <= dynamic_linear_max_tokens(K), f"{what}: at most {dynamic_linear_max_tokens(K)} tokens at K = {K}")
+    _check(x.stride(0) % 8 == 0, f"{what}: the activation row stride must be a multiple of 8")
+    _check(w_scale is None or (w_scale.dtype == torch.float32 and w_scale.numel() == N and w_scale.is_contiguous()
+                               and w_scale.device == x.device), f"{what}: w_scale must hold one fp32 scale per channel")
+    out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if M == 0 or N == 0:
+        return out
+    L = _abi.lib()
+    fn = L.llmq_linear_fp8_dynamic if fp8 else L.llmq_linear_i8_dynamic
+    st = fn(x.data_ptr(), _abi.dtype_code(x.dtype), x.stride(0), w.data_ptr(), w.stride(1), _abi.ptr(w_scale), _abi.ptr(bias),
+            _abi.dtype_code(bias.dtype) if bias is not None else _abi.BF16, out.data_ptr(), _abi.dtype_code(out_dtype),
+            out.stride(0), M, N, K, _abi.ptr(q_dump), _abi.ptr(scale_dump), _abi.ptr(acc_dump), _abi.stream_of(x))
+    _abi.check(st, what)
+    return out
+
+
+@torch.no_grad()
+def w8a8_int8_linear_dynamic_per_token(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, w_scale: torch.Tensor,
+                                       *, _q_dump=None, _scale_dump=None, _acc_dump=None) -> torch.Tensor:
+    """quantize_activation_per_token_absmax (linear_sq.py:55-65) + w8a8_int8_linear_bbf16_obf16_per_channel in one
+    launch, for up to dynamic_linear_max_tokens(K) tokens; bit-identical to the two calls.  ``x``: bf16 / fp16 [M, K];
+    ``weight``: int8 [K, N] view of an [N, K] row-major tensor; ``bias``: [N], its dtype is the output dtype."""
+    what = "w8a8_int8_linear_dynamic_per_token"
+    _check(weight.dtype == torch.int8, f"{what}: weight must be int8")
+    _check(bias is not None, f"{what}: bias is required (pass zeros for a bias-free layer)")
+    _check_bias(bias, weight, weight.size(1), (torch.bfloat16, torch.float16), what)
+    return _run_dynamic(False, x, weight, bias, w_scale, bias.dtype, _q_dump, _scale_dump, _acc_dump, what)
+
+
+@torch.no_grad()
+def f8f8bf16_linear_dynamic_per_token(x: torch.Tensor, WQ: torch.Tensor, bias: Optional[torch.Tensor],
+                                      w_scale: torch.Tensor, *, _q_dump=None, _scale_dump=None,
+                                      _acc_dump=None) -> torch.Tensor:
+    """per_token_quantize (linear_fp8.py:40-63) + cutlass_f8f8bf16_rowwise_sm89 in one launch, for up to
+    dynamic_linear_max_tokens(K) tokens; bit-identical to the two calls.  Output bf16."""
+    what = "f8f8bf16_linear_dynamic_per_token"
+    _check(WQ.dtype == torch.float8_e4m3fn, f"{what}: WQ must be float8_e4m3fn")
+    _check_bias(bias, WQ, WQ.size(1), (torch.bfloat16, torch.float32), what)
+    return _run_dynamic(True, x, WQ, bias, w_scale, torch.bfloat16, _q_dump, _scale_dump, _acc_dump, what)
