@@ -713,14 +713,32 @@ bool skinny_plan(int64_t M, int64_t N, int64_t K, int& t, int& nw) {
         return true;
     }
     if (g_force_cfg >= 0) return false;
-    // Measured on the Qwen2-7B projections against the tile kernel with split K (two launches): ahead up to 16
-    // tokens for qkv / o (7.3 / 5.6 us against 8.4 / 8.3 at one token, 8.5 / 6.5 against 9.8 / 9.3 at 16) and up to
-    // 8 tokens for down; every wavefront re-reads the activations of its K run, so the advantage shrinks with the
-    // token count, and for gate_up (N = 37888) the tile kernel already streams at 5.5 TB/s.
-    if (M > 16 || N > 8192 || (K >= 8192 && M > 8)) return false;
-    if (K < 8192 && N >= 4096) t = 2, nw = 4;
-    else t = 1, nw = 8;
-    return true;
+    // Measured on the Qwen2-7B projections with the weights coming out of HBM, against the tile kernel (with and
+    // without split K): ahead up to 16 tokens for every projection with N <= 8192 (8 tokens for a long K: every
+    // wavefront re-reads the activations of its K run), and up to 32 tokens for a short K, where the tile kernel has
+    // only N / 128 blocks to pull the weights with (o: 7.1 / 8.3 us against 14.0 / 13.1 at 17 / 32 tokens, qkv 9.4 /
+    // 10.9 against 15.7 / 15.5); a narrow N keeps the lead to 64 tokens with 16 wavefronts along K (o: 11.3 against
+    // 13.5 us).  For gate_up (N = 37888) the tile kernel already streams at 5.5 TB/s.
+    if (N > 8192) return false;
+    if (K >= 8192) {
+        if (M > 8) return false;
+        t = 1, nw = 8;
+        return true;
+    }
+    if (M <= 16) {
+        if (N >= 4096) t = 2, nw = 4;
+        else t = 1, nw = 8;
+        return true;
+    }
+    if (M <= 32) {
+        t = N >= 4096 ? 2 : 1, nw = 4;
+        return true;
+    }
+    if (N < 4096) {
+        t = 1, nw = 16;
+        return true;
+    }
+    return false;
 }
 
 // Pick the tile shape and K split with the smallest modelled time:
