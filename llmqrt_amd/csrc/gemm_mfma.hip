@@ -689,6 +689,7 @@ constexpr TileShape kShapes[] = {
     {64, 128, 128},   // 4: 4 waves x (32x64)
     {32, 128, 128},   // 5: 4 waves x (32x32), decode
     {256, 256, 128},  // 6: 8 waves x (128x64), whole 128-byte lines per row (fp8 prefill)
+    {128, 256, 128},  // 7: 8 waves x (64x64): twice the tiles of config 6 for grids that would leave CUs idle
 };
 constexpr int kNumShapes = sizeof(kShapes) / sizeof(kShapes[0]);
 
@@ -766,6 +767,7 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, double mfma_scale = 1.0, bool fp
         {3, 1, 0.27, 8.0},   // 128x128
         {4, 1, 0.15, 7.0},   // 64x128
         {5, 1, 0.10, 6.0},   // 32x128
+        {7, 1, 0.45, 8.0},   // 128x256, 8 waves
     };
     Plan best{1, 1, (int)K};
     double best_t = 1e300;
@@ -776,6 +778,9 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, double mfma_scale = 1.0, bool fp
         if (M > 128 && md.cfg == 5) continue;
         if (M > 128 && md.cfg == 4 && (M > 1024 || (int64_t)cdiv(M, 128) * cdiv(N, 128) >= 2 * kNumCu)) continue;
         if (md.cfg < 5 && M <= s.bm / 2) continue;            // mostly padding
+        // 128x256 tiles are for grids that 256x256 tiles cannot fill twice over (measured: o / down at M = 2048,
+        // gate_up at M = 512, qkv at M = 4096: 8-17 % ahead; with more tiles the big tile's lower operand traffic wins)
+        if (md.cfg == 7 && (M <= 64 || (int64_t)cdiv(M, 256) * cdiv(N, 256) >= 2 * kNumCu)) continue;
         const int64_t tiles = (int64_t)cdiv(M, s.bm) * cdiv(N, s.bn);
         for (int sp = 1; sp <= 16; sp++) {
             if (sp > 1 && (K / sp < 512 || (int64_t)M * N * sp > (int64_t)64 << 20)) break;
@@ -784,7 +789,9 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, double mfma_scale = 1.0, bool fp
             if (eff_sp != sp) continue;
             const int64_t slots = (int64_t)kNumCu * md.per_cu, blocks = tiles * sp;
             const int64_t full_rounds = blocks / slots, rest = blocks % slots;
-            const double tt = md.t_tile * mfma_scale * (fp8 && s.bk == 64 ? 1.2 : 1.0);
+            // fp8: the 64-byte K tiles run the slower register-staged loop; unsplit, config 1 is launched as the
+            // 128-byte-tile config 6 (gemm_entry), which does not
+            const double tt = md.t_tile * mfma_scale * (fp8 && s.bk == 64 && !(md.cfg == 1 && sp == 1) ? 1.2 : 1.0);
             double t = full_rounds * (kps / 64.0 * tt + md.fixed);
             if (rest) t += kps / 64.0 * tt * (0.52 + 0.48 * (double)rest / slots) + md.fixed;
             // two 64-row blocks fit a CU side by side and share its load path: between one and two blocks per CU the
@@ -842,6 +849,7 @@ int launch_shape(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, i
         case 3: return launch_cfg<GemmCfg<128, 128, 64, 2, 2, FP8, AFMT, 2, DMA && !FP8>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
         case 4: return launch_cfg<GemmCfg<64, 128, 128, 2, 2, FP8, AFMT, 2, DMA>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
         case 6: return launch_cfg<GemmCfg<256, 256, 128, 2, 4, FP8, AFMT, 1, DMA>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
+        case 7: return launch_cfg<GemmCfg<128, 256, 128, 2, 4, FP8, AFMT, 1, DMA>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
         default: return launch_cfg<GemmCfg<32, 128, 128, 1, 4, FP8, AFMT, 2, DMA>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
     }
 }

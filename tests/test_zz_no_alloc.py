@@ -59,7 +59,7 @@ def test_static_scratch_gemm_matches_workspace_gemm(cuda):
 def test_static_scratch_gemm_rejects_oversized_problems(cuda):
     from llmqrt_amd import _abi
     L = _abi.lib()
-    M, N, K = 1024, 4096, 65536
+    M, N, K = 1536, 4096, 65536
     assert L.llmq_gemm_workspace_bytes(M, N, K) > L.llmq_gemm_static_scratch_bytes()
     rc = L.llmq_gemm_w8a8_static(0x1000, K, 0x1000, K, None, None, 1.0, None, None, 0, 0.0, 0x1000, 0, N, M, N, K, None)
     assert rc == -7 and b"scratch" in L.llmq_status_string(rc)
