@@ -32,12 +32,13 @@ def dequant_matmul_token_threshold(in_features: int, out_features: int = 0) -> i
 
     The reference switches to dequantize + torch.matmul at 1024 tokens (linear_awq.py:22,47).  Here both sides are
     this library's kernels; measured on the Qwen2-7B shapes the fused path (streaming kernels up to 64 tokens, tile
-    kernel with in-loop dequantization above) is ahead up to ~380 tokens for down (K = 18944), ~500-750 for qkv / o
-    and ~1500 for gate_up (N = 37888, where the dequantizer's 70 us take longest to amortize).  Both paths are within
-    1e-2 (max relative) of dequantize-then-matmul in fp32."""
+    kernel with in-loop dequantization above) is ahead up to ~256 tokens for qkv / o (K = 3584; 34 / 29 us against
+    32 / 30), ~380 for down (K = 18944) and ~550 for gate_up (N = 37888, where the dequantizer's 70 us take longest to
+    amortize: 134 against 183 us at 256 tokens, 231 against 234 at 512).  Both paths are within 1e-2 (max relative) of
+    dequantize-then-matmul in fp32."""
     if in_features > 8192:
         return 384
-    return 1536 if out_features > 8192 else 640
+    return 576 if out_features > 8192 else 288
 
 
 def awq_linear_forward(x, qweight, qzeros, scales, w_bit=4, group_size=128, bias=None, out_features=0):
