@@ -420,22 +420,23 @@ def test_tail_split_equals_single_launch(cuda):
     the single launch that the accumulator dump selects; sampled accumulator rows exact.  FP8 gate_up at M = 4096
     (9.25 rounds) with an fp32 bias likewise."""
     from llmqrt_amd.sq_fp8_kernels import cutlass_f8f8bf16_rowwise_sm89, w8a8_int8_linear_bbf16_obf16_per_channel
-    M, N, K = 8192, 4608, 3584
     g = torch.Generator().manual_seed(77)
-    qx = torch.randint(-128, 128, (M, K), dtype=torch.int8, generator=g)
-    qw = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=g)
-    sx = torch.rand(M, generator=g) * 0.05 + 0.01
-    sw = torch.rand(N, generator=g) * 0.01 + 0.001
-    bias = torch.randn(N, generator=g).bfloat16().to(cuda)
-    a, b = qx.to(cuda), qw.to(cuda).t()
-    sxd, swd = sx.to(cuda).view(-1, 1), sw.to(cuda).view(1, -1)
-    dump = torch.empty((M, N), dtype=torch.int32, device=cuda)
-    single = w8a8_int8_linear_bbf16_obf16_per_channel(a, b, bias, sxd, swd, _acc_dump=dump)
-    split = w8a8_int8_linear_bbf16_obf16_per_channel(a, b, bias, sxd, swd)
-    assert torch.equal(split.view(torch.int16), single.view(torch.int16))
-    rows = torch.arange(3, M, M // 32)
-    assert torch.equal(dump[rows.to(cuda)].cpu(), R.int8_gemm_exact(qx[rows], qw))
-    del a, b, dump, single, split
+    for N in (4608, 4600):  # the second: a ragged last channel tile in the second part
+        M, K = 8192, 3584
+        qx = torch.randint(-128, 128, (M, K), dtype=torch.int8, generator=g)
+        qw = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=g)
+        sx = torch.rand(M, generator=g) * 0.05 + 0.01
+        sw = torch.rand(N, generator=g) * 0.01 + 0.001
+        bias = torch.randn(N, generator=g).bfloat16().to(cuda)
+        a, b = qx.to(cuda), qw.to(cuda).t()
+        sxd, swd = sx.to(cuda).view(-1, 1), sw.to(cuda).view(1, -1)
+        dump = torch.empty((M, N), dtype=torch.int32, device=cuda)
+        single = w8a8_int8_linear_bbf16_obf16_per_channel(a, b, bias, sxd, swd, _acc_dump=dump)
+        split = w8a8_int8_linear_bbf16_obf16_per_channel(a, b, bias, sxd, swd)
+        assert torch.equal(split.view(torch.int16), single.view(torch.int16)), N
+        rows = torch.arange(3, M, M // 32)
+        assert torch.equal(dump[rows.to(cuda)].cpu(), R.int8_gemm_exact(qx[rows], qw)), N
+        del a, b, dump, single, split
     M, N, K = 4096, 37888, 3584
     xq = (torch.randn(M, K, generator=g) * 0.5).to(torch.float8_e4m3fn).to(cuda)
     wq = (torch.randn(N, K, generator=g) * 0.5).to(torch.float8_e4m3fn).to(cuda)
