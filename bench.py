@@ -529,6 +529,51 @@ def details_layer(dev):
     return out
 
 
+def details_few_tokens(dev):
+    """W8A8 linears at 1 / 16 / 32 tokens with the weights coming out of HBM (rotated through > 256 MB of copies, as in
+    a model whose weights do not fit the Infinity Cache): per-token quantizer + GEMM as two launches (the few-token
+    GEMM kernel or the tile kernel, as the plan decides) against the one-launch linear that quantizes inside the GEMM
+    kernel (where the token count fits it)."""
+    from llmqrt_amd import _abi, workloads as W
+    L = _abi.lib()
+    stream_obj = torch.cuda.current_stream()
+    stream = stream_obj.cuda_stream
+    out = []
+    for pi, (pname, (K, N)) in enumerate(W.QWEN2_7B_PROJ.items()):
+        qw, ws = W.int8_weights(N, K, W.seed_for(1, 100 + pi))
+        ncopies = max(2, -(-320 * 1024 * 1024 // (N * K)))
+        copies = [qw.to(dev).clone() for _ in range(ncopies)]
+        ws = ws.to(dev)
+        row = {"proj": pname, "weight_MB": round(N * K / 1e6, 1)}
+        for M in (1, 16, 32):
+            x = W.activations(M, K, 7).to(dev)
+            q = torch.empty((M, K), dtype=torch.int8, device=dev)
+            sa = torch.empty(M, dtype=torch.float32, device=dev)
+            y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+            nws = max(int(L.llmq_gemm_workspace_bytes(M, N, K)), 16)
+            wsp = torch.empty(nws, dtype=torch.uint8, device=dev)
+
+            def two(c):
+                def f():
+                    rc = L.llmq_quant_i8_per_token(x.data_ptr(), _abi.BF16, M, K, K, q.data_ptr(), sa.data_ptr(), _abi.F32, stream)
+                    rc |= L.llmq_gemm_w8a8(q.data_ptr(), K, c.data_ptr(), K, sa.data_ptr(), ws.data_ptr(), 1.0, None, None, 0, 0.0,
+                                           y.data_ptr(), _abi.BF16, N, M, N, K, None, wsp.data_ptr(), nws, stream)
+                    return rc
+                return f
+
+            def one(c):
+                return lambda: L.llmq_linear_i8_dynamic(x.data_ptr(), _abi.BF16, K, c.data_ptr(), K, ws.data_ptr(), None, 0,
+                                                        y.data_ptr(), _abi.BF16, N, M, N, K, None, None, None, stream)
+            assert two(copies[0])() == 0
+            row[f"M{M}_quant_plus_gemm_us"] = round(batch_time_us([two(c) for c in copies], stream_obj, max(2 * ncopies, 40)), 2)
+            if M <= L.llmq_linear_dynamic_max_tokens(K):
+                assert one(copies[0])() == 0
+                row[f"M{M}_one_launch_us"] = round(batch_time_us([one(c) for c in copies], stream_obj, max(2 * ncopies, 40)), 2)
+        out.append(row)
+        del copies
+    return out
+
+
 def details_norm_quant(dev):
     """RMSNorm feeding the per-token int8 quantizer: one fused kernel against the two separate ones."""
     from llmqrt_amd import _abi, workloads as W
@@ -758,6 +803,7 @@ def main():
         result["details"]["awq_w4a16"] = awq_rows
         result["details"]["layer_stack_w8a8"] = details_layer(dev)
         result["details"]["rmsnorm_quant_i8"] = details_norm_quant(dev)
+        result["details"]["w8a8_few_tokens_weights_from_hbm"] = details_few_tokens(dev)
 
     print(json.dumps(result))
 
