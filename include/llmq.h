@@ -243,8 +243,10 @@ size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 /* Tuning / test hook with no counterpart in the reference: force the kernel variant of
  * llmq_awq_gemm for every later call of this process: v = 1 or 2 words per lane of the streaming
  * kernel in 16-token slabs, 5 or 6 = streaming kernel with 2 or 4 token tiles per wavefront,
- * 3, 7 or 4 = tile kernel with 64x128, 128x128 or 256x256 tiles (any M), 0 = heuristic; the cross-block K split
- * (0 = heuristic); the wavefronts per block along K of the streaming kernel (4 or 8; 0 = heuristic).
+ * 3, 7 or 4 = tile kernel with 64x128, 128x128 or 256x256 tiles (any M), 8 .. 11 = the few-token kernel
+ * (M <= 16; 128- / 256-byte row segments, one / two stages ahead), 0 = heuristic; the cross-block K split
+ * (0 = heuristic); the wavefronts per block along K of the streaming kernel (4 or 8), or the K slices
+ * inside a block of the few-token kernel (2 or 4, v = 8 only); 0 = heuristic.
  * Process-global, not thread-safe. */
 int llmq_awq_force_plan(int v, int splits, int k_waves);
 

@@ -20,25 +20,11 @@
 //   * fp32 accumulation in the MFMA; the 4 wavefronts of a block split the block's K range and
 //     are summed through LDS in a fixed order; a K split across blocks goes through an fp32
 //     workspace and a finishing kernel, again in a fixed order (results are deterministic).
+#include "awq_plans.h"
 #include "llmq_common.h"
 
 namespace llmq {
 
-// Tile kernel for many tokens (awq_tile.hip).
-struct AwqTilePlan { int cfg, splits, k_per_split; };
-AwqTilePlan make_awq_tile_plan(int64_t M, int64_t N, int64_t K, int force_cfg, int force_splits);
-int launch_awq_tile(const AwqTilePlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
-                    const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K, int G,
-                    hipStream_t st);
-
-// Decode kernel for up to 16 tokens (awq_decode.hip).
-struct AwqDecodePlan { int cs, pd, splits, groups_per_block; };
-bool awq_decode_supported(int64_t M, int64_t N, int64_t K, int64_t group);
-AwqDecodePlan make_awq_decode_plan(int64_t M, int64_t N, int64_t K, int force_cs, int force_pd, int force_splits);
-size_t awq_decode_workspace_bytes(const AwqDecodePlan& p, int64_t M, int64_t N);
-int launch_awq_decode(const AwqDecodePlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
-                      const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K,
-                      hipStream_t st);
 
 namespace {
 
@@ -751,11 +737,11 @@ inline bool decode_path(int64_t M, int64_t group) { return M <= 64 && group == 1
 // partial sums of the K split grow with the token count; 6 for a wide N, which needs no K split: gate_up at 5 tokens
 // 19.3 against 22.5 us).
 inline bool decode16_path(int64_t M, int64_t N, int64_t K, int64_t group) {
-    return ((g_force_v == 0 && M <= (K >= 8192 ? 2 : (N >= 16384 ? 6 : 4))) || (g_force_v >= 8 && g_force_v <= 11)) && awq_decode_supported(M, N, K, group);
+    return ((g_force_v == 0 && M <= (K >= 8192 ? 8 : (N >= 16384 ? 6 : 4))) || (g_force_v >= 8 && g_force_v <= 11)) && awq_decode_supported(M, N, K, group);
 }
 inline AwqDecodePlan decode16_plan(int64_t M, int64_t N, int64_t K) {
     const int cs = g_force_v >= 8 ? ((g_force_v & 1) ? 4 : 2) : 0, pd = g_force_v >= 8 ? (g_force_v >= 10 ? 2 : 1) : 0;
-    return make_awq_decode_plan(M, N, K, cs, pd, g_force_splits);
+    return make_awq_decode_plan(M, N, K, cs, pd, g_force_splits, g_force_kw);
 }
 
 // More than 64 tokens go to the tile kernel (weights dequantized once per token tile on their way into LDS);

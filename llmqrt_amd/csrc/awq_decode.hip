@@ -24,11 +24,10 @@
 #include <atomic>
 #include <type_traits>
 
+#include "awq_plans.h"
 #include "llmq_common.h"
 
 namespace llmq {
-
-struct AwqDecodePlan { int cs, pd, splits, groups_per_block; };
 
 namespace {
 
@@ -125,28 +124,41 @@ __device__ __forceinline__ void finish_split_tile(const float* ptile, int M, int
     }
 }
 
-template <int CS, int PD, int RM>  // RM: token rows per lane that can be live (min(M, 4))
-__global__ __launch_bounds__(CS * kWave, 3) void awq_decode_kernel(
+// RM: token rows per lane that can be live (min(M, 4)).  KS: K slices inside the block - KS sets of CS wavefronts, each
+// with its own LDS stages, take consecutive shares of the block's groups (KS x the bytes in flight per block at the
+// same number of cross-block arrivals) and add their sums through LDS in slice order before the block publishes.
+template <int CS, int PD, int RM, int KS>
+__global__ __launch_bounds__(CS * KS * kWave, KS == 4 ? 2 : 3) void awq_decode_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, const uint32_t* __restrict__ qw,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qz, const uint16_t* __restrict__ bias,
     uint16_t* __restrict__ out, float* partials, unsigned int* tickets, int M, int N, int K, int gpb, int tiles_n) {
-    constexpr int NT = CS * kWave, SEGW = 16 * CS, SEGQ = SEGW / 4;  // words / 16-byte pieces per tile row
-    constexpr int RPL = NT / SEGQ;                                   // rows one block-wide load covers (16)
+    constexpr int NS = CS * kWave, NT = NS * KS;       // threads per slice / per block
+    constexpr int SEGW = 16 * CS, SEGQ = SEGW / 4;     // words / 16-byte pieces per tile row
+    constexpr int RPL = NS / SEGQ;                     // rows one slice-wide load covers (16)
     constexpr int LOADS = kStageRows / RPL;                          // 16-byte loads per thread and stage (4)
     constexpr int STRIDE = SEGW + 4;  // LDS row stride in words: keeps 16-byte alignment, spreads rows 8 apart over banks
     static_assert(RPL == 16 && LOADS == 4, "a stage is four block-wide loads");
     constexpr int XSTRIDE = 36;       // LDS row stride of the activation tile in words (64 k = 32 words + 4)
-    __shared__ __attribute__((aligned(16))) uint32_t lds[2][kStageRows * STRIDE];
-    __shared__ __attribute__((aligned(16))) uint32_t ldx_s[2][16 * XSTRIDE];  // 16 tokens x 64 k of fp16 per stage
+    __shared__ __attribute__((aligned(16))) uint32_t lds_all[KS][2][kStageRows * STRIDE];
+    __shared__ __attribute__((aligned(16))) uint32_t ldx_all[KS][2][16 * XSTRIDE];  // 16 tokens x 64 k of fp16 per stage
 
-    const int tid = threadIdx.x, lane = tid & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave_b = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int slice = wave_b / CS, wave = wave_b % CS;  // wavefront-uniform
+    const int tid = threadIdx.x - slice * NS;           // thread index inside the slice
+    uint32_t (*lds)[kStageRows * STRIDE] = lds_all[slice];
+    uint32_t (*ldx_s)[16 * XSTRIDE] = ldx_all[slice];
     const int li = lane & 15, kb = lane >> 4;
     const int Nw = N >> 3, Nq = Nw >> 2;
     const int tile = blockIdx.x % tiles_n, ks = blockIdx.x / tiles_n;
     const int ngroups = K / kGroup;
-    const int g_begin = ks * gpb, g_end = min(ngroups, g_begin + gpb);
-    const int nst = 2 * (g_end - g_begin);
+    const int bg_begin = ks * gpb, bg_end = min(ngroups, bg_begin + gpb);  // the block's groups
+    const int per_slice = (bg_end - bg_begin + KS - 1) / KS;
+    const int g_first = min(bg_begin + slice * per_slice, bg_end), g_end = min(bg_end, g_first + per_slice);
+    const int nst = 2 * (g_end - g_first);          // this slice's stages (0 when the block has fewer groups than slices)
+    const int nst_block = 2 * per_slice;            // stages the block steps through (barriers are block-wide)
+    const int g_begin = min(g_first, ngroups - 1);  // addressing base: stays inside the matrix for an empty slice
+    const int g_last = max(g_end - 1, g_begin);
 
     // ---- global -> register mapping of the cooperative tile load
     const int ld_row = tid / SEGQ, ld_seg = tid % SEGQ;
@@ -172,7 +184,7 @@ __global__ __launch_bounds__(CS * kWave, 3) void awq_decode_kernel(
     u4 s_next;
     // every load is unconditional: indices past the block's K range re-read its last stage / group
     auto load_stage = [&](int s, Stage& d) __attribute__((always_inline)) {
-        s = min(s, nst - 1);
+        s = min(s, max(nst - 1, 0));
         const u4* p = wbase + (int64_t)s * kStageRows * Nq;
         d.w0 = p[0];
         d.w1 = p[(int64_t)RPL * Nq];
@@ -181,7 +193,7 @@ __global__ __launch_bounds__(CS * kWave, 3) void awq_decode_kernel(
         if (x_loader) d.x0 = *reinterpret_cast<const u4*>(xbase + s * (kStageRows * 2));
     };
     auto load_group = [&](int g) __attribute__((always_inline)) {
-        g = min(g, g_end - 1);
+        g = min(g, g_last);
         z_next = qz[(int64_t)g * Nw + cwc];
         s_next = *reinterpret_cast<const u4*>(scales + (int64_t)g * N + 8 * cwc);
     };
@@ -219,6 +231,10 @@ __global__ __launch_bounds__(CS * kWave, 3) void awq_decode_kernel(
         }
         load_stage(st + PD, cur);
         lds_barrier();
+        if (KS > 1 && st >= nst) {  // a slice with fewer stages than the block's longest: barriers only
+            __builtin_amdgcn_sched_barrier(0);
+            return;
+        }
 #pragma unroll
         for (int c2 = 0; c2 < 2; c2++) {
             const uint32_t* lp = tile_lds + (32 * c2 + 8 * kb) * STRIDE + 16 * wave + li;
@@ -280,7 +296,7 @@ __global__ __launch_bounds__(CS * kWave, 3) void awq_decode_kernel(
 
     // stages alternate between the PD register sets; nst is even, PD is 1 or 2
 #pragma unroll 1
-    for (int st = 0; st < nst; st += 2) {
+    for (int st = 0; st < nst_block; st += 2) {
         stage_body(st, sa);
         if constexpr (PD == 2) stage_body(st + 1, sb);
         else stage_body(st + 1, sa);
@@ -302,7 +318,7 @@ __global__ __launch_bounds__(CS * kWave, 3) void awq_decode_kernel(
         }
         *reinterpret_cast<uint4*>(out + (int64_t)m * N + nn) = make_uint4(o[0], o[1], o[2], o[3]);
     };
-    if (splits == 1) {
+    if (KS == 1 && splits == 1) {
         if (!col_ok) return;
 #pragma unroll
         for (int r = 0; r < RM; r++) {
@@ -314,18 +330,29 @@ __global__ __launch_bounds__(CS * kWave, 3) void awq_decode_kernel(
         return;
     }
     constexpr int TILE_CH = SEGW * 8;  // channels per tile
-    float* ptile = reinterpret_cast<float*>(&lds[0][0]);  // [M][TILE_CH] fp32, reuses the weight stages
+    float* ptile = reinterpret_cast<float*>(&lds_all[0][0][0]);  // [M][TILE_CH] fp32, reuses the weight stages
     static_assert(2 * kStageRows * STRIDE >= 16 * TILE_CH, "the partial tile fits in the weight stages");
     __syncthreads();  // every wavefront is done reading the last stage
 #pragma unroll
-    for (int r = 0; r < RM; r++) {
-        const int m = 4 * kb + r;
-        if (m >= M) continue;
-        float4* dst = reinterpret_cast<float4*>(ptile + m * TILE_CH + (16 * wave + li) * 8);
-        dst[0] = make_float4(y[0][r], y[1][r], y[2][r], y[3][r]);
-        dst[1] = make_float4(y[4][r], y[5][r], y[6][r], y[7][r]);
+    for (int sl = 0; sl < KS; sl++) {  // slice 0 writes its sums, the others add theirs in slice order
+        if (sl == slice) {
+#pragma unroll
+            for (int r = 0; r < RM; r++) {
+                const int m = 4 * kb + r;
+                if (m >= M) continue;
+                float4* dst = reinterpret_cast<float4*>(ptile + m * TILE_CH + (16 * wave + li) * 8);
+                float4 a = make_float4(y[0][r], y[1][r], y[2][r], y[3][r]), b = make_float4(y[4][r], y[5][r], y[6][r], y[7][r]);
+                if (sl > 0) {
+                    const float4 pa = dst[0], pb = dst[1];
+                    a = make_float4(pa.x + a.x, pa.y + a.y, pa.z + a.z, pa.w + a.w);
+                    b = make_float4(pb.x + b.x, pb.y + b.y, pb.z + b.z, pb.w + b.w);
+                }
+                dst[0] = a;
+                dst[1] = b;
+            }
+        }
+        __syncthreads();
     }
-    __syncthreads();
     finish_split_tile<TILE_CH, NT>(ptile, M, N, tile, ks, splits, partials, tickets, bias, out);
 }
 
@@ -337,26 +364,33 @@ bool awq_decode_supported(int64_t M, int64_t N, int64_t K, int64_t group) {
     return M >= 1 && M <= 16 && group == kGroup && (N % 32) == 0 && (K % kGroup) == 0 && N / 256 <= kTicketRing / kTicketStride;
 }
 
-// Column tile width (CS wavefronts = 16*CS words), prefetch depth and K split.  Measured on the Qwen2-7B shapes:
-// 128-byte row segments (CS = 2) with one stage in flight beat the wider tile and the deeper prefetch everywhere;
-// about 2048 wavefronts fill the chip, but a block should keep at least two groups (pipeline fill), a column tile
-// at most ~40 arrivals (its ticket is one memory word: arrivals serialize at ~50 ns each), and the fp32 partial
-// sums, written through and read back coherently, at most an eighth of the weight bytes.
-AwqDecodePlan make_awq_decode_plan(int64_t M, int64_t N, int64_t K, int force_cs, int force_pd, int force_splits) {
+// Column tile width (CS wavefronts = 16*CS words), prefetch depth, K slices per block and K split.  Measured on the
+// Qwen2-7B shapes: 128-byte row segments (CS = 2) with one stage in flight beat the wider tile and the deeper prefetch
+// everywhere; about 2048 wavefronts fill the chip, but a block should keep at least two groups (pipeline fill), a
+// column tile at most ~40 arrivals (its ticket is one memory word: arrivals serialize at ~50 ns each), and the fp32
+// partial sums, written through and read back coherently, at most an eighth of the weight bytes.  Where the column
+// tiles alone cannot fill the chip, K slices inside the block raise the bytes in flight without more arrivals:
+// 2 slices for a short K (qkv / o at one token 7.5 -> 6.7 us, at four 10.8 -> 8.4), 4 slices of about 3 groups each
+// for a long K (down 13.9 -> 12.0 us); with enough column tiles (gate_up) slices only cost (17.1 -> 18.9 us).
+AwqDecodePlan make_awq_decode_plan(int64_t M, int64_t N, int64_t K, int force_cs, int force_pd, int force_splits, int force_ks) {
     const int groups = (int)(K / kGroup), Nw = (int)(N / 8);
     AwqDecodePlan p;
     p.cs = force_cs > 0 ? force_cs : 2;
+    p.pd = force_pd > 0 ? force_pd : 1;
     const int strips = cdiv_d(Nw, 16);  // wavefront-wide column strips
+    p.ks = strips >= 128 ? 1 : (K >= 8192 ? 4 : 2);
+    if (force_ks == 1 || force_ks == 2 || force_ks == 4) p.ks = force_ks;
+    if (p.cs != 2 || p.pd != 1) p.ks = 1;  // the slices exist for the 128-byte tile with one stage ahead only
     int s = cdiv_d(2048, strips);
     if (s > 40) s = 40;
     if (s > groups / 2) s = groups / 2;
+    if (p.ks == 4 && s > cdiv_d(groups, 11)) s = cdiv_d(groups, 11);  // slices of 3, 3, 3 and 2 groups
     if (s > K / (128 * M)) s = (int)(K / (128 * M));  // 2 * S * M * N * 4 <= K * N / 2 / 8
     if (force_splits > 0) s = force_splits;
     if (s > groups) s = groups;
     if (s < 1) s = 1;
     p.groups_per_block = cdiv_d(groups, s);
     p.splits = cdiv_d(groups, p.groups_per_block);
-    p.pd = force_pd > 0 ? force_pd : 1;
     return p;
 }
 
@@ -396,19 +430,21 @@ int launch_awq_decode(const AwqDecodePlan& p, const uint16_t* x, int64_t ldx, co
         const int rc = ticket_slots(tiles_n, &tickets);
         if (rc != LLMQ_OK) return rc;
     }
-#define LLMQ_DECODE_RM(CS_, PD_, RM_)                                                                                 \
-    hipLaunchKernelGGL((awq_decode_kernel<CS_, PD_, RM_>), grid, dim3(CS_ * kWave), 0, st, x, ldx, qw, scales, qz, bias, \
-                       out, ws, tickets, M, N, K, p.groups_per_block, tiles_n)
-#define LLMQ_DECODE(CS_, PD_)                  \
-    do {                                       \
-        if (M == 1) LLMQ_DECODE_RM(CS_, PD_, 1);      \
-        else if (M == 2) LLMQ_DECODE_RM(CS_, PD_, 2); \
-        else LLMQ_DECODE_RM(CS_, PD_, 4);             \
+#define LLMQ_DECODE_RM(CS_, PD_, RM_, KS_)                                                                            \
+    hipLaunchKernelGGL((awq_decode_kernel<CS_, PD_, RM_, KS_>), grid, dim3(CS_ * KS_ * kWave), 0, st, x, ldx, qw, scales, \
+                       qz, bias, out, ws, tickets, M, N, K, p.groups_per_block, tiles_n)
+#define LLMQ_DECODE(CS_, PD_, KS_)                         \
+    do {                                                   \
+        if (M == 1) LLMQ_DECODE_RM(CS_, PD_, 1, KS_);      \
+        else if (M == 2) LLMQ_DECODE_RM(CS_, PD_, 2, KS_); \
+        else LLMQ_DECODE_RM(CS_, PD_, 4, KS_);             \
     } while (0)
-    if (p.cs == 4 && p.pd == 2) LLMQ_DECODE(4, 2);
-    else if (p.cs == 4) LLMQ_DECODE(4, 1);
-    else if (p.pd == 2) LLMQ_DECODE(2, 2);
-    else LLMQ_DECODE(2, 1);
+    if (p.cs == 4 && p.pd == 2) LLMQ_DECODE(4, 2, 1);
+    else if (p.cs == 4) LLMQ_DECODE(4, 1, 1);
+    else if (p.pd == 2) LLMQ_DECODE(2, 2, 1);
+    else if (p.ks == 4) LLMQ_DECODE(2, 1, 4);
+    else if (p.ks == 2) LLMQ_DECODE(2, 1, 2);
+    else LLMQ_DECODE(2, 1, 1);
 #undef LLMQ_DECODE
 #undef LLMQ_DECODE_RM
     return launch_status();

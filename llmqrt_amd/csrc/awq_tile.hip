@@ -20,6 +20,7 @@
 // the end of K is zeroed when it is written to LDS, rows past M and channels past N are never stored.
 #include <type_traits>
 
+#include "awq_plans.h"
 #include "llmq_common.h"
 
 namespace llmq {
@@ -297,9 +298,6 @@ int launch_tile(const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16
 }
 
 }  // namespace
-
-// Tile shapes: 0 = 64 tokens x 128 channels (4 wavefronts), 1 = 256 x 256 (8 wavefronts), 2 = 128 x 128 (4 wavefronts).
-struct AwqTilePlan { int cfg, splits, k_per_split; };  // also declared in awq.hip
 
 AwqTilePlan make_awq_tile_plan(int64_t M, int64_t N, int64_t K, int force_cfg, int force_splits) {
     AwqTilePlan p;

@@ -238,6 +238,29 @@ def test_decode_kernel_every_variant_and_split(cuda, force_awq_plan, variant, sp
     assert torch.equal(out, out2), "deterministic"
 
 
+@pytest.mark.parametrize("slices", [2, 4])
+@pytest.mark.parametrize("splits", [0, 1, 3])
+@pytest.mark.parametrize("M,K,N", DECODE_SHAPES + [(8, 18944, 3584), (5, 640, 288)])
+def test_decode_kernel_k_slices_inside_the_block(cuda, force_awq_plan, slices, splits, M, K, N):
+    """K slices inside a block (2 or 4 sets of wavefronts with their own LDS stages, added in slice order): against
+    the oracle and deterministic, fused and split along K, with bias; covers blocks with fewer groups than slices
+    (K = 128: one group for four slices; K = 640 in 3 splits: 2 + 2 + 1 groups) and the long K of `down`."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    qw, qz, s = W.awq_weights(N, K, 17 * M + N)
+    x = W.activations(M, K, 19 * M + K, dtype=torch.float16, outliers=False)
+    bias = (0.1 * torch.randn(N, generator=torch.Generator().manual_seed(M))).half() if splits != 1 else None
+    ref = R.awq_gemm(x, qw, qz, s, 128)
+    if bias is not None:
+        ref = (ref.float() + bias.float()).half()
+    force_awq_plan(8, splits, slices)
+    args = (x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda))
+    out = awq_gemm_triton(*args, split_k_iters=8, bias=None if bias is None else bias.to(cuda))
+    assert rel_err(out, ref) <= REL_TOL, (slices, splits, M, K, N)
+    out2 = awq_gemm_triton(*args, split_k_iters=8, bias=None if bias is None else bias.to(cuda))
+    assert torch.equal(out, out2), "deterministic"
+
+
 def test_decode_kernel_extreme_nibbles_and_zero_tokens(cuda, force_awq_plan):
     """All-15 weights against zero points 0 and all-0 weights against zero points 15 (the largest |q - z|), and a
     token block whose rows past M must not leak into the result."""
