@@ -731,13 +731,13 @@ DecodePlan make_decode_plan(int64_t M, int64_t N, int64_t K) {
 // The streaming kernel handles up to 64 tokens per weight pass as up to 4 slabs of 16.
 inline bool decode_path(int64_t M, int64_t group) { return M <= 64 && group == 128; }
 
-// The LDS-staged decode kernel (one launch, in-kernel K-split reduction) serves the first few tokens, where it is
-// ahead of the register-streaming kernel; llmq_awq_force_plan 8..11 picks its tile width and prefetch depth for any
-// M <= 16, 1 / 2 / 5 / 6 keep the register-streaming kernel.  Measured crossover: 4 tokens (2 for a long K, where the
-// partial sums of the K split grow with the token count; 6 for a wide N, which needs no K split: gate_up at 5 tokens
-// 19.3 against 22.5 us).
+// The LDS-staged decode kernel (one launch, in-kernel K-split reduction) serves up to 16 tokens wherever its shape
+// conditions hold (group 128, N a multiple of 32); with the K slices and splits of make_awq_decode_plan it is level
+// with or ahead of the register-streaming kernel on every measured shape (o at 16 tokens 10.4 against 10.1 us is the
+// one tie; qkv 10.7 against 11.3, gate_up 21.9 against 24.1, down 17.3 against 18.2).  llmq_awq_force_plan 8..11
+// picks its tile width and prefetch depth, 1 / 2 / 5 / 6 keep the register-streaming kernel.
 inline bool decode16_path(int64_t M, int64_t N, int64_t K, int64_t group) {
-    return ((g_force_v == 0 && M <= (K >= 8192 ? 8 : (N >= 16384 ? 6 : 4))) || (g_force_v >= 8 && g_force_v <= 11)) && awq_decode_supported(M, N, K, group);
+    return ((g_force_v == 0 && M <= 16) || (g_force_v >= 8 && g_force_v <= 11)) && awq_decode_supported(M, N, K, group);
 }
 inline AwqDecodePlan decode16_plan(int64_t M, int64_t N, int64_t K) {
     const int cs = g_force_v >= 8 ? ((g_force_v & 1) ? 4 : 2) : 0, pd = g_force_v >= 8 ? (g_force_v >= 10 ? 2 : 1) : 0;

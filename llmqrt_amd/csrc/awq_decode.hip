@@ -21,6 +21,7 @@
 //     arrives last at a column tile adds them in split order and writes the output: one launch, results
 //     independent of scheduling.  Arrivals are counted in a ring of self-resetting tickets that the library owns
 //     (a zero-initialised static device array; every call takes fresh slots, so concurrent calls do not share any).
+#include <algorithm>
 #include <atomic>
 #include <type_traits>
 
@@ -365,31 +366,44 @@ bool awq_decode_supported(int64_t M, int64_t N, int64_t K, int64_t group) {
 }
 
 // Column tile width (CS wavefronts = 16*CS words), prefetch depth, K slices per block and K split.  Measured on the
-// Qwen2-7B shapes: 128-byte row segments (CS = 2) with one stage in flight beat the wider tile and the deeper prefetch
-// everywhere; about 2048 wavefronts fill the chip, but a block should keep at least two groups (pipeline fill), a
-// column tile at most ~40 arrivals (its ticket is one memory word: arrivals serialize at ~50 ns each), and the fp32
-// partial sums, written through and read back coherently, at most an eighth of the weight bytes.  Where the column
-// tiles alone cannot fill the chip, K slices inside the block raise the bytes in flight without more arrivals:
-// 2 slices for a short K (qkv / o at one token 7.5 -> 6.7 us, at four 10.8 -> 8.4), 4 slices of about 3 groups each
-// for a long K (down 13.9 -> 12.0 us); with enough column tiles (gate_up) slices only cost (17.1 -> 18.9 us).
+// Qwen2-7B shapes (weights streamed from HBM): 128-byte row segments (CS = 2) with one stage in flight beat the wider
+// tile and the deeper prefetch everywhere.  About 2048 wavefronts fill the chip, but a column tile should see at most
+// ~40 arrivals (its ticket is one memory word: arrivals serialize at ~50 ns each), and the fp32 partial sums, written
+// through and read back coherently by the one block that finishes a tile, grow with splits x tokens: the more tokens,
+// the fewer blocks along K and the more K slices inside a block (bytes in flight without more arrivals).
+//   wide N (column tiles alone nearly fill the chip; gate_up): one slice and ~2048 wavefronts up to 4 tokens
+//     (17-20 us), blocks of 6 groups at 5-6 tokens (19.0), 2 slices x 5 groups at 7-8 (19.2), beyond that 4 slices
+//     and no split across blocks (21.9 at 16 tokens; the register-streaming kernel needs 24.1);
+//   long K (down): 4 slices of ~3 groups (12.0 us at one token against 13.9 with one slice; 17.3 at 16);
+//   short K, narrow N (qkv, o): 2 slices of one group up to 4 tokens (6.7 us at one token against 7.5; 8.4 at 4
+//     against 10.8), 4 slices of one group beyond (8.9 at 8, 10.7 at 16 tokens).
 AwqDecodePlan make_awq_decode_plan(int64_t M, int64_t N, int64_t K, int force_cs, int force_pd, int force_splits, int force_ks) {
     const int groups = (int)(K / kGroup), Nw = (int)(N / 8);
     AwqDecodePlan p;
     p.cs = force_cs > 0 ? force_cs : 2;
     p.pd = force_pd > 0 ? force_pd : 1;
     const int strips = cdiv_d(Nw, 16);  // wavefront-wide column strips
-    p.ks = strips >= 128 ? 1 : (K >= 8192 ? 4 : 2);
+    int s = cdiv_d(2048, strips);       // enough wavefronts
+    if (s > 40) s = 40;
+    if (strips >= 128) {
+        if (M <= 4) p.ks = 1, s = (int)std::min<int64_t>(s, std::max<int64_t>(groups / M, 1));
+        else if (M <= 6) p.ks = 1, s = std::min(s, cdiv_d(groups, 6));
+        else if (M <= 8) p.ks = 2, s = std::min(s, cdiv_d(groups, 10));
+        else p.ks = 4, s = 1;
+    } else if (K >= 8192) {
+        p.ks = 4, s = std::min(s, cdiv_d(groups, 11));
+    } else if (M <= 4) {
+        p.ks = 2, s = (int)std::min<int64_t>(std::min(s, groups / 2), std::max<int64_t>(groups / M, 1));
+    } else {
+        p.ks = 4, s = std::min(s, cdiv_d(groups, 4));
+    }
     if (force_ks == 1 || force_ks == 2 || force_ks == 4) p.ks = force_ks;
     if (p.cs != 2 || p.pd != 1) p.ks = 1;  // the slices exist for the 128-byte tile with one stage ahead only
-    int s = cdiv_d(2048, strips);
-    if (s > 40) s = 40;
-    if (s > groups / 2) s = groups / 2;
-    if (p.ks == 4 && s > cdiv_d(groups, 11)) s = cdiv_d(groups, 11);  // slices of 3, 3, 3 and 2 groups
-    if (s > K / (128 * M)) s = (int)(K / (128 * M));  // 2 * S * M * N * 4 <= K * N / 2 / 8
     if (force_splits > 0) s = force_splits;
     if (s > groups) s = groups;
     if (s < 1) s = 1;
     p.groups_per_block = cdiv_d(groups, s);
+    if (force_splits <= 0) p.groups_per_block = cdiv_d(p.groups_per_block, p.ks) * p.ks;  // equal shares for the slices
     p.splits = cdiv_d(groups, p.groups_per_block);
     return p;
 }
