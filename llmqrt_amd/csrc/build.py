@@ -16,7 +16,9 @@ OUT_DIR = HERE.parent / "lib"
 OBJ_DIR = OUT_DIR / "obj"
 LIB = OUT_DIR / "libllmq_gfx950.so"
 MICROBENCH_LIB = OUT_DIR / "libllmq_microbench_gfx950.so"  # hardware microbenchmarks for `bench.py --micro`; not the product
-SOURCES = ["abi.hip", "quant.hip", "gemm_mfma.hip", "gemm_skinny.hip", "linear_fused.hip", "awq.hip", "awq_decode.hip", "awq_tile.hip"]
+# the tile GEMM is instantiated per operand format in four translation units (the long poles of the build), listed first
+SOURCES = ["gemm_tile_i8.hip", "gemm_tile_fp8.hip", "gemm_tile_fp8_e5m2.hip", "gemm_tile_f16.hip", "gemm_mfma.hip", "abi.hip",
+           "quant.hip", "gemm_skinny.hip", "linear_fused.hip", "awq.hip", "awq_decode.hip", "awq_tile.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -49,7 +51,7 @@ def _link(lib: pathlib.Path, objs) -> None:
 
 def build(verbose: bool = True) -> pathlib.Path:
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
-    with concurrent.futures.ThreadPoolExecutor(max_workers=4) as ex:
+    with concurrent.futures.ThreadPoolExecutor(max_workers=6) as ex:
         objs = list(ex.map(_compile, SOURCES + ["microbench.hip"]))
     _link(LIB, objs[:-1])
     _link(MICROBENCH_LIB, objs[-1:])
