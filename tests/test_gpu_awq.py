@@ -261,6 +261,48 @@ def test_decode_kernel_k_slices_inside_the_block(cuda, force_awq_plan, slices, s
     assert torch.equal(out, out2), "deterministic"
 
 
+@pytest.mark.parametrize("M,K,N", [(4, 3584, 4608), (16, 18944, 3584)])
+def test_decode_kernel_in_a_hip_graph(cuda, M, K, N):
+    """The few-token kernel ends its K split inside the launch with arrival tickets that return to zero; a captured
+    launch replays on the slots it was captured with.  Every replay, with fresh activations and eager calls (which
+    take other slots) in between, must reproduce the eager result bit for bit."""
+    from llmqrt_amd import _abi, workloads as W
+    L = _abi.lib()
+    qw, qz, s = (t.to(cuda) for t in W.awq_weights(N, K, 77 + M))
+    x = W.activations(M, K, 700, dtype=torch.float16, outliers=False).to(cuda)
+    out = torch.empty((M, N), dtype=torch.float16, device=cuda)
+    nws = L.llmq_awq_gemm_workspace_bytes(M, N, K)
+    assert nws > 0, "the shapes are meant to exercise the K split"
+    wsp = torch.empty(nws, dtype=torch.uint8, device=cuda)
+
+    def run(stream):
+        rc = L.llmq_awq_gemm(x.data_ptr(), K, qw.data_ptr(), s.data_ptr(), qz.data_ptr(), None, out.data_ptr(), M, N, K,
+                             128, wsp.data_ptr(), nws, stream)
+        assert rc == 0
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        run(side.cuda_stream)   # first call on the device outside the capture (looks up the ticket ring once)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            run(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    main = torch.cuda.current_stream().cuda_stream
+    for rep in range(4):
+        x.copy_(W.activations(M, K, 710 + rep, dtype=torch.float16, outliers=False).to(cuda))
+        run(main)
+        torch.cuda.synchronize()
+        eager = out.clone()
+        out.zero_()
+        wsp.fill_(0xFF)          # the workspace contents must not matter
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep}"
+    ref = R.awq_gemm(x.cpu(), qw.cpu(), qz.cpu(), s.cpu(), 128)
+    assert rel_err(out, ref) <= REL_TOL
+
+
 def test_decode_kernel_extreme_nibbles_and_zero_tokens(cuda, force_awq_plan):
     """All-15 weights against zero points 0 and all-0 weights against zero points 15 (the largest |q - z|), and a
     token block whose rows past M must not leak into the result."""
