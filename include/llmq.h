@@ -228,8 +228,8 @@ int llmq_gemm_num_configs(void);
 /* out[m,n] = fp16( sum_k x[m,k] * fp16((q[k,n] - z[k/G,n]) * s[k/G,n]) + bias[n] ), fp32
  * accumulation in a fixed order (deterministic, unlike the reference's fp16 atomics).
  * x: fp16 [M,K] (ldx >= K, K % 32 == 0); out: fp16 [M,N] contiguous; bias: fp16 [N] or NULL.
- * Up to 64 tokens a streaming kernel runs (for up to 16 tokens and group 128 the weights enter the
- * matrix core unrounded, exact (q - z) * s in fp32, instead of rounded to fp16 first); above 64 tokens
+ * Up to 64 tokens a streaming kernel runs (for group 128 the weights enter the matrix core
+ * unrounded, exact (q - z) * s in fp32, instead of rounded to fp16 first); above 64 tokens
  * an fp16 tile GEMM dequantizes the weights on their way into LDS.  All are within 1e-2 of the
  * dequantize-then-matmul math.
  * workspace: >= llmq_awq_gemm_workspace_bytes(M,N,K) bytes, 16-byte aligned, contents irrelevant. */
@@ -244,9 +244,9 @@ size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * llmq_awq_gemm for every later call of this process: v = 1 or 2 words per lane of the streaming
  * kernel in 16-token slabs, 5 or 6 = streaming kernel with 2 or 4 token tiles per wavefront,
  * 3, 7 or 4 = tile kernel with 64x128, 128x128 or 256x256 tiles (any M), 8 .. 11 = the few-token kernel
- * (M <= 16; 128- / 256-byte row segments, one / two stages ahead), 0 = heuristic; the cross-block K split
+ * (M <= 64; 128- / 256-byte row segments, one / two stages ahead), 0 = heuristic; the cross-block K split
  * (0 = heuristic); the wavefronts per block along K of the streaming kernel (4 or 8), or the K slices
- * inside a block of the few-token kernel (2 or 4, v = 8 only); 0 = heuristic.
+ * inside a block of the few-token kernel (1, 2 or 4, v = 8 only); 0 = heuristic.
  * Process-global, not thread-safe. */
 int llmq_awq_force_plan(int v, int splits, int k_waves);
 

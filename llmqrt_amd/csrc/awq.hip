@@ -719,7 +719,7 @@ DecodePlan make_decode_plan(int64_t M, int64_t N, int64_t K) {
     // instead of one (gate_up at 64 tokens: 58 -> 56.6 us from HBM, 52 -> 43 us with cache-resident weights).
     p.v = (p.ms == 1 && M <= 16 && Nw % 2 == 0 && Nw / 32 >= 128) ? 2 : 1;
     if (p.ms == 1 && (g_force_v == 1 || (g_force_v == 2 && Nw % 2 == 0))) p.v = g_force_v;
-    p.kw = (g_force_kw > 0 && p.v == 1 && p.ms == 1) ? g_force_kw : 4;
+    p.kw = ((g_force_kw == 4 || g_force_kw == 8) && p.v == 1 && p.ms == 1) ? g_force_kw : 4;
     const int ntiles = cdiv(Nw, 16 * p.v);
     int splits = g_force_splits > 0 ? g_force_splits : (ntiles >= 128 ? 1 : cdiv(200, ntiles));  // measured optimum: ~200 blocks
     if (splits > groups / p.kw) splits = groups / p.kw;  // at least one group per wavefront
@@ -731,13 +731,13 @@ DecodePlan make_decode_plan(int64_t M, int64_t N, int64_t K) {
 // The streaming kernel handles up to 64 tokens per weight pass as up to 4 slabs of 16.
 inline bool decode_path(int64_t M, int64_t group) { return M <= 64 && group == 128; }
 
-// The LDS-staged decode kernel (one launch, in-kernel K-split reduction) serves up to 16 tokens wherever its shape
-// conditions hold (group 128, N a multiple of 32); with the K slices and splits of make_awq_decode_plan it is level
-// with or ahead of the register-streaming kernel on every measured shape (o at 16 tokens 10.4 against 10.1 us is the
-// one tie; qkv 10.7 against 11.3, gate_up 21.9 against 24.1, down 17.3 against 18.2).  llmq_awq_force_plan 8..11
-// picks its tile width and prefetch depth, 1 / 2 / 5 / 6 keep the register-streaming kernel.
+// The LDS-staged decode kernel (one launch, in-kernel K-split reduction) serves up to 64 tokens (slabs of 16) wherever
+// its shape conditions hold (group 128, N a multiple of 32); with the K slices and splits of make_awq_decode_plan it
+// is level with or ahead of the register-streaming kernel on every measured shape (o at 16 tokens 10.4 against 10.1 us
+// is the one tie; at 64 tokens qkv 14.4 against 19.8, gate_up 43.8 against 57.1, down 28.8 against 31.1).
+// llmq_awq_force_plan 8..11 picks its tile width and prefetch depth, 1 / 2 / 5 / 6 keep the register-streaming kernel.
 inline bool decode16_path(int64_t M, int64_t N, int64_t K, int64_t group) {
-    return ((g_force_v == 0 && M <= 16) || (g_force_v >= 8 && g_force_v <= 11)) && awq_decode_supported(M, N, K, group);
+    return ((g_force_v == 0 && M <= 64) || (g_force_v >= 8 && g_force_v <= 11)) && awq_decode_supported(M, N, K, group);
 }
 inline AwqDecodePlan decode16_plan(int64_t M, int64_t N, int64_t K) {
     const int cs = g_force_v >= 8 ? ((g_force_v & 1) ? 4 : 2) : 0, pd = g_force_v >= 8 ? (g_force_v >= 10 ? 2 : 1) : 0;
@@ -766,7 +766,7 @@ void launch_awq(const AwqPlan& p, const uint16_t* x, int64_t ldx, const uint32_t
 using namespace llmq;
 
 extern "C" int llmq_awq_force_plan(int v, int splits, int k_waves) {
-    if (v < 0 || v > 11 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 2 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
+    if (v < 0 || v > 11 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 1 && k_waves != 2 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
     g_force_v = v;
     g_force_splits = splits;
     g_force_kw = k_waves;
@@ -780,7 +780,7 @@ extern "C" size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
         const AwqTilePlan t = tile_plan(M, N, K);
         if (t.splits > 1) total = (size_t)t.splits * M * N * sizeof(float);
     }
-    if (M <= 16 && awq_decode_supported(M, N, K, 128)) {
+    if (awq_decode_supported(M, N, K, 128)) {
         const size_t need = awq_decode_workspace_bytes(decode16_plan(M, N, K), M, N);
         if (need > total) total = need;
     }

@@ -1,4 +1,4 @@
-// AWQ W4A16 decode kernel: up to 16 tokens, group size 128, N a multiple of 32.
+// AWQ W4A16 decode kernel: up to 64 tokens in slabs of 16, group size 128, N a multiple of 32.
 //
 // The op is a stream of half a byte per weight out of HBM, so the kernel is laid out around the memory
 // system first.  Measured on MI355X with a pure-load kernel over the [K, N/8] int32 weight matrix: a
@@ -44,7 +44,7 @@ __host__ __device__ constexpr int rev_nibble_d(int j) { return ((j & 1) << 2) | 
 
 // Cross-block end of a K split, shared by the decode kernels.  On entry `ptile` (LDS, [M][TILE_CH] fp32) holds this
 // block's partial sums for column tile `tile` and every thread of the block has passed a barrier after writing it.
-// Every block publishes its tile to partials[ks][M][N]; the block that arrives last at the tile adds the splits in
+// Every block publishes its tile to partials[ks] (planes of `plane` floats, rows of N); the block that arrives last at the tile adds the splits in
 // split order (so the result does not depend on which block that is), adds the bias and writes the output.
 // Cross-block visibility without cache-wide fences (a device-scope release fence writes back the whole L2 of the
 // XCD: measured at ~100 us per launch): the partial sums are stored and loaded with the device-coherent cache
@@ -57,8 +57,8 @@ constexpr int kTicketStride = 64;  // in 4-byte words
 constexpr int kTicketRing = 1 << 18;  // words in the ring of tickets
 template <int TILE_CH, int NT>
 __device__ __forceinline__ void finish_split_tile(const float* ptile, int M, int N, int tile, int ks, int splits,
-                                                  float* partials, unsigned int* tickets, const uint16_t* bias,
-                                                  uint16_t* out) {
+                                                  float* partials, int64_t plane, unsigned int* tickets,
+                                                  const uint16_t* bias, uint16_t* out) {
     const int tid = threadIdx.x;
     const int tile_n0 = tile * TILE_CH;                  // first channel of the tile
     const int tile_q = min(TILE_CH, N - tile_n0) >> 2;   // its width in units of 4 channels (N % 32 == 0)
@@ -84,7 +84,7 @@ __device__ __forceinline__ void finish_split_tile(const float* ptile, int M, int
     for (int idx = tid; idx < M * tile_q; idx += NT) {
         const int m = idx / tile_q, c4 = idx - m * tile_q;
         const v4f v = *reinterpret_cast<const v4f*>(ptile + m * TILE_CH + 4 * c4);
-        float* dst = partials + ((int64_t)ks * M + m) * N + tile_n0 + 4 * c4;
+        float* dst = partials + (int64_t)ks * plane + (int64_t)m * N + tile_n0 + 4 * c4;
         asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's coherent stores have completed
@@ -101,7 +101,7 @@ __device__ __forceinline__ void finish_split_tile(const float* ptile, int M, int
     for (int idx = tid; idx < M * tile_q; idx += NT) {
         const int m = idx / tile_q, nn = tile_n0 + 4 * (idx - m * tile_q);
         const float* src = partials + (int64_t)m * N + nn;
-        const int64_t sstride = (int64_t)M * N;
+        const int64_t sstride = plane;
         v4f acc = {0.f, 0.f, 0.f, 0.f};
         for (int sp = 0; sp < splits; sp += 8) {  // eight coherent loads in flight, added in split order
             v4f t0, t1, t2, t3, t4, t5, t6, t7;
@@ -132,7 +132,8 @@ template <int CS, int PD, int RM, int KS>
 __global__ __launch_bounds__(CS * KS * kWave, KS == 4 ? 2 : 3) void awq_decode_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, const uint32_t* __restrict__ qw,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qz, const uint16_t* __restrict__ bias,
-    uint16_t* __restrict__ out, float* partials, unsigned int* tickets, int M, int N, int K, int gpb, int tiles_n) {
+    uint16_t* __restrict__ out, float* partials, unsigned int* tickets, int Mtot, int N, int K, int gpb, int tiles_n,
+    int splits, int slabs) {
     constexpr int NS = CS * kWave, NT = NS * KS;       // threads per slice / per block
     constexpr int SEGW = 16 * CS, SEGQ = SEGW / 4;     // words / 16-byte pieces per tile row
     constexpr int RPL = NS / SEGQ;                     // rows one slice-wide load covers (16)
@@ -151,7 +152,22 @@ __global__ __launch_bounds__(CS * KS * kWave, KS == 4 ? 2 : 3) void awq_decode_k
     uint32_t (*ldx_s)[16 * XSTRIDE] = ldx_all[slice];
     const int li = lane & 15, kb = lane >> 4;
     const int Nw = N >> 3, Nq = Nw >> 2;
-    const int tile = blockIdx.x % tiles_n, ks = blockIdx.x / tiles_n;
+    // Work item = (column tile, K split); token slab = 16 tokens.  With several slabs the slabs of a work item sit next
+    // to each other on one XCD (flat block ids go round-robin over the 8 XCDs), so the weights cross the fabric once
+    // and the other slabs find them in that XCD's L2; blocks past the padded end leave at once.
+    int work = blockIdx.x, slab = 0;
+    if (slabs > 1) {
+        const int q = blockIdx.x >> 3;
+        slab = q % slabs;
+        work = (q / slabs) * 8 + (blockIdx.x & 7);
+        if (work >= tiles_n * splits) return;  // block-uniform, before any barrier
+    }
+    const int tile = work % tiles_n, ks = work / tiles_n;
+    const int M = min(16, Mtot - 16 * slab);  // tokens of this slab
+    x += (int64_t)slab * 16 * ldx;
+    out += (int64_t)slab * 16 * N;
+    if (partials) partials += (int64_t)slab * 16 * N;
+    if (tickets) tickets += kTicketStride * tiles_n * slab;
     const int ngroups = K / kGroup;
     const int bg_begin = ks * gpb, bg_end = min(ngroups, bg_begin + gpb);  // the block's groups
     const int per_slice = (bg_end - bg_begin + KS - 1) / KS;
@@ -304,7 +320,6 @@ __global__ __launch_bounds__(CS * KS * kWave, KS == 4 ? 2 : 3) void awq_decode_k
     }
 
     // ---- store: lane (word column li, quarter kb) holds tokens 4*kb + r for its 8 channels
-    const int splits = gridDim.x / tiles_n;
     const int n = 8 * cw;
     auto finish8 = [&](const float* v, int m, int nn) __attribute__((always_inline)) {  // 8 channels -> fp16 (+ bias), one 16-byte store
         uint32_t o[4];
@@ -354,7 +369,7 @@ __global__ __launch_bounds__(CS * KS * kWave, KS == 4 ? 2 : 3) void awq_decode_k
         }
         __syncthreads();
     }
-    finish_split_tile<TILE_CH, NT>(ptile, M, N, tile, ks, splits, partials, tickets, bias, out);
+    finish_split_tile<TILE_CH, NT>(ptile, M, N, tile, ks, splits, partials, (int64_t)Mtot * N, tickets, bias, out);
 }
 
 inline int cdiv_d(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
@@ -362,7 +377,7 @@ inline int cdiv_d(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 }  // namespace
 
 bool awq_decode_supported(int64_t M, int64_t N, int64_t K, int64_t group) {
-    return M >= 1 && M <= 16 && group == kGroup && (N % 32) == 0 && (K % kGroup) == 0 && N / 256 <= kTicketRing / kTicketStride;
+    return M >= 1 && M <= 64 && group == kGroup && (N % 32) == 0 && (K % kGroup) == 0 && 4 * (N / 256 + 1) <= kTicketRing / kTicketStride;
 }
 
 // Column tile width (CS wavefronts = 16*CS words), prefetch depth, K slices per block and K split.  Measured on the
@@ -376,7 +391,10 @@ bool awq_decode_supported(int64_t M, int64_t N, int64_t K, int64_t group) {
 //     and no split across blocks (21.9 at 16 tokens; the register-streaming kernel needs 24.1);
 //   long K (down): 4 slices of ~3 groups (12.0 us at one token against 13.9 with one slice; 17.3 at 16);
 //   short K, narrow N (qkv, o): 2 slices of one group up to 4 tokens (6.7 us at one token against 7.5; 8.4 at 4
-//     against 10.8), 4 slices of one group beyond (8.9 at 8, 10.7 at 16 tokens).
+//     against 10.8), 4 slices of one group beyond (8.9 at 8, 10.7 at 16 tokens);
+//   17-64 tokens run as slabs of 16 tokens that share the weights through one XCD's L2: qkv 12.3 us at 32 and 14.4
+//     at 64 tokens (register-streaming kernel + finish kernel: 13.8 / 19.8), o 11.7 / 13.5 (13.1 / 17.5), gate_up
+//     33.2 / 43.8 (39.2 / 57.1), down 21.1 / 28.8 (22.4 / 31.1).
 AwqDecodePlan make_awq_decode_plan(int64_t M, int64_t N, int64_t K, int force_cs, int force_pd, int force_splits, int force_ks) {
     const int groups = (int)(K / kGroup), Nw = (int)(N / 8);
     AwqDecodePlan p;
@@ -385,7 +403,16 @@ AwqDecodePlan make_awq_decode_plan(int64_t M, int64_t N, int64_t K, int force_cs
     const int strips = cdiv_d(Nw, 16);  // wavefront-wide column strips
     int s = cdiv_d(2048, strips);       // enough wavefronts
     if (s > 40) s = 40;
-    if (strips >= 128) {
+    if (M > 16) {
+        // Token slabs multiply the blocks: keep them all resident at once (4 slices = 92 KB of LDS, one block per CU;
+        // 2 slices = 46 KB, three) - a second round of blocks costs more than any split gains.
+        const int slabs = cdiv_d(M, 16), tiles = cdiv_d(strips, 2) * slabs;
+        p.ks = tiles <= 256 ? 4 : 2;
+        const int fit = std::max(1, (p.ks == 4 ? 256 : 768) / tiles);
+        if (strips >= 128) s = p.ks == 4 ? 1 : std::min(fit, 2);
+        else if (K >= 8192) s = std::min(cdiv_d(groups, 11), fit);
+        else s = std::min(cdiv_d(groups, 4), fit);
+    } else if (strips >= 128) {
         if (M <= 4) p.ks = 1, s = (int)std::min<int64_t>(s, std::max<int64_t>(groups / M, 1));
         else if (M <= 6) p.ks = 1, s = std::min(s, cdiv_d(groups, 6));
         else if (M <= 8) p.ks = 2, s = std::min(s, cdiv_d(groups, 10));
@@ -438,15 +465,16 @@ int launch_awq_decode(const AwqDecodePlan& p, const uint16_t* x, int64_t ldx, co
                       const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K,
                       hipStream_t st) {
     const int tiles_n = cdiv_d(N / 8, 16 * p.cs);
-    const dim3 grid((unsigned)(tiles_n * p.splits));
+    const int slabs = cdiv_d(M, 16), work = tiles_n * p.splits;
+    const dim3 grid((unsigned)(slabs == 1 ? work : cdiv_d(work, 8) * 8 * slabs));
     unsigned int* tickets = nullptr;
     if (p.splits > 1) {
-        const int rc = ticket_slots(tiles_n, &tickets);
+        const int rc = ticket_slots(tiles_n * slabs, &tickets);
         if (rc != LLMQ_OK) return rc;
     }
 #define LLMQ_DECODE_RM(CS_, PD_, RM_, KS_)                                                                            \
     hipLaunchKernelGGL((awq_decode_kernel<CS_, PD_, RM_, KS_>), grid, dim3(CS_ * KS_ * kWave), 0, st, x, ldx, qw, scales, \
-                       qz, bias, out, ws, tickets, M, N, K, p.groups_per_block, tiles_n)
+                       qz, bias, out, ws, tickets, M, N, K, p.groups_per_block, tiles_n, p.splits, slabs)
 #define LLMQ_DECODE(CS_, PD_, KS_)                         \
     do {                                                   \
         if (M == 1) LLMQ_DECODE_RM(CS_, PD_, 1, KS_);      \

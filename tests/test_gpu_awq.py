@@ -261,7 +261,31 @@ def test_decode_kernel_k_slices_inside_the_block(cuda, force_awq_plan, slices, s
     assert torch.equal(out, out2), "deterministic"
 
 
-@pytest.mark.parametrize("M,K,N", [(4, 3584, 4608), (16, 18944, 3584)])
+@pytest.mark.parametrize("plan", [(0, 0, 0), (8, 0, 2), (8, 3, 4), (8, 1, 1), (8, 5, 2)])
+@pytest.mark.parametrize("M,K,N", [(17, 1024, 288), (33, 512, 4608), (50, 3584, 1024), (64, 896, 4864), (40, 18944, 3584),
+                                   (64, 3584, 37888), (31, 128, 32)])
+def test_decode_kernel_token_slabs(cuda, force_awq_plan, plan, M, K, N):
+    """17-64 tokens through the few-token kernel as slabs of 16 tokens (a ragged last slab; column-tile x split counts
+    that are not multiples of 8, so that padded blocks exit; more blocks than fit at once): the automatic plan and
+    forced slices / splits, against the oracle, with bias and a row stride larger than K; deterministic."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    qw, qz, s = W.awq_weights(N, K, 23 * M + N)
+    x = W.activations(M, 2 * K, 29 * M + K, dtype=torch.float16, outliers=False)
+    bias = (0.1 * torch.randn(N, generator=torch.Generator().manual_seed(M))).half()
+    ref = (R.awq_gemm(x[:, :K], qw, qz, s, 128).float() + bias.float()).half()
+    force_awq_plan(*plan)
+    xd = x.to(cuda)[:, :K]
+    assert xd.stride(0) == 2 * K
+    args = (xd, qw.to(cuda), s.to(cuda), qz.to(cuda))
+    out = awq_gemm_triton(*args, split_k_iters=8, bias=bias.to(cuda))
+    assert out.shape == (M, N) and out.dtype == torch.float16
+    assert rel_err(out, ref) <= REL_TOL, (plan, M, K, N)
+    out2 = awq_gemm_triton(*args, split_k_iters=8, bias=bias.to(cuda))
+    assert torch.equal(out, out2), "deterministic"
+
+
+@pytest.mark.parametrize("M,K,N", [(4, 3584, 4608), (16, 18944, 3584), (48, 3584, 4608)])
 def test_decode_kernel_in_a_hip_graph(cuda, M, K, N):
     """The few-token kernel ends its K split inside the launch with arrival tickets that return to zero; a captured
     launch replays on the slots it was captured with.  Every replay, with fresh activations and eager calls (which
