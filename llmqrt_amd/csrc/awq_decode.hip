@@ -377,7 +377,9 @@ inline int cdiv_d(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 }  // namespace
 
 bool awq_decode_supported(int64_t M, int64_t N, int64_t K, int64_t group) {
-    return M >= 1 && M <= 64 && group == kGroup && (N % 32) == 0 && (K % kGroup) == 0 && 4 * (N / 256 + 1) <= kTicketRing / kTicketStride;
+    // a call's tickets (one per column tile and token slab) must fit in half of the ring
+    return M >= 1 && M <= 64 && group == kGroup && (N % 32) == 0 && (K % kGroup) == 0 &&
+           2 * ((M + 15) / 16) * (N / 256 + 1) <= kTicketRing / kTicketStride;
 }
 
 // Column tile width (CS wavefronts = 16*CS words), prefetch depth, K slices per block and K split.  Measured on the
@@ -441,8 +443,10 @@ size_t awq_decode_workspace_bytes(const AwqDecodePlan& p, int64_t M, int64_t N) 
 }
 
 // Arrival tickets: a ring of counters, all zero between calls (each returns to zero with its last arrival).  A call
-// takes tiles_n consecutive slots at a cursor that only moves forward, so two calls can only meet on a slot if more
-// than kTicketRing / tiles_n later calls were issued while the first had still not run.  One copy per GPU.
+// reserves a run of consecutive slots at a cursor that only moves forward; a reservation that would cross the end of
+// the ring is dropped and taken again (the next one starts near the front and cannot cross: a run is at most half
+// the ring), so no two reservations ever overlap until the cursor has gone once around, i.e. two calls can only meet
+// on a slot if more than kTicketRing / run later calls were issued while the first had still not run.  One copy per GPU.
 static __device__ unsigned int g_ticket_ring[kTicketRing];
 static unsigned int* g_ticket_ptr[64] = {};  // device address of each GPU's copy, looked up once per device
 
@@ -455,8 +459,12 @@ static int ticket_slots(int tiles_n, unsigned int** out) {
         g_ticket_ptr[dev] = static_cast<unsigned int*>(p);  // benign if two threads race: same address
     }
     static std::atomic<unsigned long long> cursor{0};
-    unsigned long long at = cursor.fetch_add((unsigned long long)tiles_n * kTicketStride, std::memory_order_relaxed) % kTicketRing;
-    if (at + (unsigned long long)tiles_n * kTicketStride > kTicketRing) at = 0;  // a run that would cross the end starts over at the front
+    const unsigned long long run = (unsigned long long)tiles_n * kTicketStride;
+    if (2 * run > kTicketRing) return LLMQ_ERR_SHAPE;  // awq_decode_supported keeps callers below this
+    unsigned long long at;
+    do {
+        at = cursor.fetch_add(run, std::memory_order_relaxed) % kTicketRing;
+    } while (at + run > kTicketRing);
     *out = g_ticket_ptr[dev] + at;
     return LLMQ_OK;
 }
