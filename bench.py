@@ -34,11 +34,11 @@ if ROOT not in sys.path:
 # WRITE_SIZE of two `rocprofv3 --pmc` runs of `bench.py --roofline-only`, each scaled by what the same
 # counter reads for the 256 MiB calibration copy (2.000 and 1.000); see
 # profiles/gemm_w8a8_int8_mfma_prefill_qwen2_7b.md.  A measured constant: counters cannot be read from here.
-ROOFLINE_TRAFFIC_BYTES = 608364616
+ROOFLINE_TRAFFIC_BYTES = 607520869
 # The same for the FP8 launches (bench.py --fp8-only, profiles/gemm_fp8_mfma_prefill_qwen2_7b.md) and the W4A16
 # decode launches at M <= 16 (bench.py --awq-only, profiles/awq_gemv_w4a16_decode_qwen2_7b.md); None = not measured.
-FP8_TRAFFIC_BYTES = 303875862
-W4A16_TRAFFIC_BYTES = 33791236
+FP8_TRAFFIC_BYTES = 304239907
+W4A16_TRAFFIC_BYTES = 33791464
 CPU_BASELINE_REPS = 12        # bounded CPU sample: about 10-15 s of host work
 PEAK_INT8_TOPS = 5033.0   # dense int8 MFMA peak of MI355X, TOP/s (256 CU x 2.4 GHz x 8192 op/clk)
 PEAK_FP8_TFLOPS = 5033.0  # dense fp8 MFMA peak

@@ -247,6 +247,7 @@ size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * (M <= 64; 128- / 256-byte row segments, one / two stages ahead), 0 = heuristic; the cross-block K split
  * (0 = heuristic); the wavefronts per block along K of the streaming kernel (4 or 8), or the K slices
  * inside a block of the few-token kernel (1, 2 or 4, v = 8 only); 0 = heuristic.
+ * v + 32 keeps the tile kernel's register-staged activation loads (default: straight into LDS when K % 64 == 0).
  * Process-global, not thread-safe. */
 int llmq_awq_force_plan(int v, int splits, int k_waves);
 

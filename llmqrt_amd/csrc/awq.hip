@@ -766,6 +766,9 @@ void launch_awq(const AwqPlan& p, const uint16_t* x, int64_t ldx, const uint32_t
 using namespace llmq;
 
 extern "C" int llmq_awq_force_plan(int v, int splits, int k_waves) {
+    const int staged = v >= 0 ? (v & 32) : 0;  // + 32: the tile kernel keeps its register-staged activation loads
+    if (v >= 0) v &= ~32;
+    set_awq_tile_direct_loads(staged ? 0 : 1);
     if (v < 0 || v > 11 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 1 && k_waves != 2 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
     g_force_v = v;
     g_force_splits = splits;

@@ -12,6 +12,7 @@ namespace llmq {
 // Tile shapes: 0 = 64 tokens x 128 channels (4 wavefronts), 1 = 256 x 256 (8 wavefronts), 2 = 128 x 128 (4 wavefronts).
 struct AwqTilePlan { int cfg, splits, k_per_split; };
 AwqTilePlan make_awq_tile_plan(int64_t M, int64_t N, int64_t K, int force_cfg, int force_splits);
+void set_awq_tile_direct_loads(int on);  // 0: register-staged activation loads only
 int launch_awq_tile(const AwqTilePlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
                     const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K, int G,
                     hipStream_t st);

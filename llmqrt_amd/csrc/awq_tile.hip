@@ -66,7 +66,10 @@ __device__ __forceinline__ void tile_coords(int bid, int nblk, int tiles_m, int 
     tn = (pid % width) / gsize;
 }
 
-template <class C>
+// ADMA: the activation tile goes global -> LDS directly (global_load_lds_dwordx4: a lane names its own 16 global
+// bytes, a wavefront's 64 pieces land back to back in LDS, so the swizzle is applied on the fetch side); needs whole
+// K tiles.  The weights always pass through registers: they are dequantized on the way.
+template <class C, bool ADMA>
 __global__ __launch_bounds__(C::NT) void awq_tile_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, const uint32_t* __restrict__ qw,
     const uint16_t* __restrict__ scales, const uint32_t* __restrict__ qz, const uint16_t* __restrict__ bias,
@@ -104,14 +107,31 @@ __global__ __launch_bounds__(C::NT) void awq_tile_kernel(
     uint32_t magic = 0x64006400u;
     asm volatile("" : "+v"(magic));  // opaque: (u & mask) | magic stays one v_and_or_b32
 
-    uint4 a_reg[C::A_LOADS];
+    uint4 a_reg[ADMA ? 1 : C::A_LOADS];
     uint32_t w_reg[8], z_reg;
     uint4 s_reg;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem_raw);
+    const uint32_t wave_off = (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 1024u;
+    // direct load of the activation tile kt into `stage`: slot i of a thread lands at chunk (tid + i * NT) of the stage,
+    // i.e. row ld_row + i * ROWS_STEP, chunk slot ld_c, which holds global chunk ld_c ^ swizzle(row)
+    auto issue_a = [&](int kt, int stage) {
+        const int ktc = max(min(kt, ktiles - 1), 0) * kBK;
+#pragma unroll
+        for (int i = 0; i < C::A_LOADS; i++) {
+            const int row = ld_row + i * ROWS_STEP;
+            const int gc = ld_c ^ (((row >> 1) ^ (row >> 3)) & 7);
+            const uint16_t* src = a_base + a_off(i) + ktc + gc * 8;
+            const uint32_t m0v = lds_base + (uint32_t)stage * (C::STAGE_CHUNKS * 16u) + wave_off + (uint32_t)i * (C::NT * 16u);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0v), "v"(src) : "memory", "m0");
+        }
+    };
     auto load_tile = [&](int kt) {
         const int ktc = max(min(kt, ktiles - 1), 0) * kBK;
-        const int ka = min(ktc + ld_c * 8, klen - 8);
+        if constexpr (!ADMA) {
+            const int ka = min(ktc + ld_c * 8, klen - 8);
 #pragma unroll
-        for (int i = 0; i < C::A_LOADS; i++) a_reg[i] = *reinterpret_cast<const uint4*>(a_base + a_off(i) + ka);
+            for (int i = 0; i < C::A_LOADS; i++) a_reg[i] = *reinterpret_cast<const uint4*>(a_base + a_off(i) + ka);
+        }
         const int kw = k_begin + min(ktc + wo * 8, klen - 8);
         const uint32_t* wp = qw + (int64_t)kw * Nw + cw;
 #pragma unroll
@@ -123,11 +143,13 @@ __global__ __launch_bounds__(C::NT) void awq_tile_kernel(
     auto store_tile = [&](int stage, int kt) {
         uint4* sA = lds + stage * C::STAGE_CHUNKS;
         uint4* sB = sA + C::BM * kCPR;
-        const uint32_t keep_a = (kt < ktiles && kt * kBK + ld_c * 8 < klen) ? 0xffffffffu : 0u;
+        if constexpr (!ADMA) {
+            const uint32_t keep_a = (kt < ktiles && kt * kBK + ld_c * 8 < klen) ? 0xffffffffu : 0u;
 #pragma unroll
-        for (int i = 0; i < C::A_LOADS; i++) {
-            const uint4 v = a_reg[i];
-            sA[st_a(i)] = make_uint4(v.x & keep_a, v.y & keep_a, v.z & keep_a, v.w & keep_a);
+            for (int i = 0; i < C::A_LOADS; i++) {
+                const uint4 v = a_reg[i];
+                sA[st_a(i)] = make_uint4(v.x & keep_a, v.y & keep_a, v.z & keep_a, v.w & keep_a);
+            }
         }
         const uint32_t keep_w = (kt < ktiles && kt * kBK + wo * 8 < klen) ? 0xffffffffu : 0u;
         const uint32_t sw[4] = {s_reg.x, s_reg.y, s_reg.z, s_reg.w};
@@ -203,20 +225,50 @@ __global__ __launch_bounds__(C::NT) void awq_tile_kernel(
 
     // ---- main loop: tile kt is computed from LDS stage kt & 1 while tile kt + 1 waits in registers
     // (dequantized and written to the other stage behind the MFMAs) and tile kt + 2 is in flight ------
-    load_tile(0);
-    store_tile(0, 0);
-    load_tile(1);
-    lds_barrier();
+    if constexpr (ADMA) {
+        // The activation tile kt + 1 is requested at the top of step kt, into the stage that every wavefront finished
+        // reading before the last barrier, and has the step's MFMAs to land.  The wait below covers it: it sits before
+        // the step's own register loads are issued (a past-the-end tile re-reads the last one into a stage that an
+        // all-zero weight tile multiplies, or that nobody reads).
+        auto landed = [] { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+        issue_a(0, 0);
+        load_tile(0);
+        store_tile(0, 0);
+        landed();
+        load_tile(1);
+        lds_barrier();
 #pragma unroll 1
-    for (int kt = 0; kt < ktiles; kt += 2) {
-        tile_mfma(0);
-        store_tile(1, kt + 1);
-        load_tile(kt + 2);
+        for (int kt = 0; kt < ktiles; kt += 2) {
+            issue_a(kt + 1, 1);
+            tile_mfma(0);
+            store_tile(1, kt + 1);
+            landed();
+            load_tile(kt + 2);
+            lds_barrier();
+            issue_a(kt + 2, 0);
+            tile_mfma(1);  // an odd tile count computes one all-zero tile here
+            store_tile(0, kt + 2);
+            landed();
+            load_tile(kt + 3);
+            lds_barrier();
+        }
+        landed();  // nothing may still be landing in LDS when the block ends
+    } else {
+        load_tile(0);
+        store_tile(0, 0);
+        load_tile(1);
         lds_barrier();
-        tile_mfma(1);  // an odd tile count computes one all-zero tile here
-        store_tile(0, kt + 2);
-        load_tile(kt + 3);
-        lds_barrier();
+#pragma unroll 1
+        for (int kt = 0; kt < ktiles; kt += 2) {
+            tile_mfma(0);
+            store_tile(1, kt + 1);
+            load_tile(kt + 2);
+            lds_barrier();
+            tile_mfma(1);  // an odd tile count computes one all-zero tile here
+            store_tile(0, kt + 2);
+            load_tile(kt + 3);
+            lds_barrier();
+        }
     }
 
     // ---- epilogue: lane = token l32; register r = channel 8 (r / 4) + 4 khalf + r % 4 of the 32-wide tile
@@ -275,11 +327,11 @@ __global__ __launch_bounds__(C::NT) void awq_tile_kernel(
 
 inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
-template <class C>
-int launch_tile(const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales, const uint32_t* qz,
+template <class C, bool ADMA>
+int launch_tile_impl(const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales, const uint32_t* qz,
                 const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K, int G, int splits, int kps,
                 hipStream_t st) {
-    auto kernel = awq_tile_kernel<C>;
+    auto kernel = awq_tile_kernel<C, ADMA>;
     if (C::LDS_BYTES > 64 * 1024) {
         // per device: the attribute belongs to the loaded code object of the current device
         static bool raised[64] = {};
@@ -297,7 +349,21 @@ int launch_tile(const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16
     return launch_status();
 }
 
+int g_awq_tile_dma = 1;  // 0 keeps the register-staged activation loads (tuning / test hook)
+
+template <class C>
+int launch_tile(const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales, const uint32_t* qz,
+                const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K, int G, int splits, int kps,
+                hipStream_t st) {
+    // the direct loads cannot zero a ragged K tail; their global addresses must be 16-byte aligned
+    const bool dma = g_awq_tile_dma && K % kBK == 0 && kps % kBK == 0 && (ldx & 7) == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+    return dma ? launch_tile_impl<C, true>(x, ldx, qw, scales, qz, bias, out, ws, M, N, K, G, splits, kps, st)
+               : launch_tile_impl<C, false>(x, ldx, qw, scales, qz, bias, out, ws, M, N, K, G, splits, kps, st);
+}
+
 }  // namespace
+
+void set_awq_tile_direct_loads(int on) { g_awq_tile_dma = on; }
 
 AwqTilePlan make_awq_tile_plan(int64_t M, int64_t N, int64_t K, int force_cfg, int force_splits) {
     AwqTilePlan p;

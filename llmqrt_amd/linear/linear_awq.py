@@ -31,13 +31,14 @@ def dequant_matmul_token_threshold(in_features: int, out_features: int = 0) -> i
     fused kernels on MI355X.
 
     The reference switches to dequantize + torch.matmul at 1024 tokens (linear_awq.py:22,47).  Here both sides are
-    this library's kernels; measured on the Qwen2-7B shapes the fused path (streaming kernels up to 64 tokens, tile
-    kernel with in-loop dequantization above) is ahead up to ~256 tokens for qkv / o (K = 3584; 34 / 29 us against
-    32 / 30), ~380 for down (K = 18944) and ~550 for gate_up (N = 37888, where the dequantizer's 70 us take longest to
-    amortize: 134 against 183 us at 256 tokens, 231 against 234 at 512).  Both paths are within 1e-2 (max relative) of
+    this library's kernels; measured on the Qwen2-7B shapes (us, fused / dequantize + GEMM) the fused path (few-token
+    kernel up to 64 tokens, tile kernel with in-loop dequantization above) is ahead up to ~256 tokens for qkv / o
+    (K = 3584; o 31 / 33 at 256 tokens, 36 / 34 at 320), ~224 for down (K = 18944; 79 / 83 at 192, 92 / 90 at 256,
+    122 / 102 at 320) and ~550 for gate_up (N = 37888, where the dequantizer's 63 us take longest to amortize:
+    138 / 185 at 256 tokens, 222 / 237 at 512, 264 / 247 at 640).  Both paths are within 1e-2 (max relative) of
     dequantize-then-matmul in fp32."""
     if in_features > 8192:
-        return 384
+        return 256
     return 576 if out_features > 8192 else 288
 
 
