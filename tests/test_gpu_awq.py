@@ -176,6 +176,26 @@ def test_tile_kernel_every_shape_and_split(cuda, force_awq_plan, tile, splits, M
     assert torch.equal(out, out2), "deterministic"
 
 
+@pytest.mark.parametrize("tile", [3, 4, 7])
+@pytest.mark.parametrize("M,K,N,G,xstride", [(65, 64, 8, 64, 64), (257, 512, 264, 512, 1024), (130, 3584, 4608, 128, 3584),
+                                            (300, 1088, 520, 32, 1096), (600, 1024, 1000, 128, 1024)])
+def test_tile_kernel_direct_loads_equal_register_staging(cuda, force_awq_plan, tile, M, K, N, G, xstride):
+    """With K a multiple of 64 the tile kernel fetches its activation tiles straight into LDS; variant + 32 keeps the
+    register-staged loop.  Same products, same order: equal on every element, for every tile shape, ragged token /
+    channel edges, several token tiles, and a row stride larger than K."""
+    from llmqrt_amd import workloads as W
+    from llmqrt_amd.awq_kernels import awq_gemm_triton
+    qw, qz, s = W.awq_weights(N, K, 9 * M + N, group=G)
+    x = W.activations(M, xstride, 10 * M + K, dtype=torch.float16, outliers=False).to(cuda)[:, :K]
+    args = (x, qw.to(cuda), s.to(cuda), qz.to(cuda))
+    force_awq_plan(tile, 0)
+    direct = awq_gemm_triton(*args, split_k_iters=8)
+    force_awq_plan(tile + 32, 0)
+    staged = awq_gemm_triton(*args, split_k_iters=8)
+    assert torch.equal(direct.view(torch.int16), staged.view(torch.int16))
+    assert rel_err(direct, R.awq_gemm(x.cpu(), qw, qz, s, G)) <= REL_TOL
+
+
 def test_tile_kernel_prefill_size(cuda):
     """1024 tokens of the Qwen2-7B qkv projection through the default plan (256x256 tiles)."""
     from llmqrt_amd import workloads as W
