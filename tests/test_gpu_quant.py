@@ -12,7 +12,10 @@ def _acts(M, K, seed, dtype):
     return W.activations(M, K, seed, dtype=dtype)
 
 
-SHAPES = [(1, 896), (16, 896), (7, 3584), (128, 3584), (33, 18944), (3, 8), (5, 24576), (2, 40960)]
+# the last four take the wavefront-per-row kernels (256 rows or more of at most 1024 elements): ragged row counts,
+# one and two chunks per lane, rows shorter than a wavefront
+SHAPES = [(1, 896), (16, 896), (7, 3584), (128, 3584), (33, 18944), (3, 8), (5, 24576), (2, 40960),
+          (258, 896), (1027, 1024), (300, 8), (257, 520)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
