@@ -36,6 +36,7 @@ __global__ __launch_bounds__(kThreads) void quant_rows_kernel(
 
     uint4 cache[NC > 0 ? NC : 1];
     float s;
+    bool fin = false;  // block-uniform: the absmax behind the scale is finite, so no quotient can be NaN
     if (SCALE == SCALE_ROW) {
         float amax = 0.f;
         if (NC > 0) {
@@ -51,11 +52,13 @@ __global__ __launch_bounds__(kThreads) void quant_rows_kernel(
         }
         amax = block_max<kNW>(amax, smem);
         s = scale_from_amax<DT, MODE>(amax);
+        fin = amax < __builtin_inff() && s > 0.f;  // (the fp8 floor rounds to 0 in fp16: an all-zero row has scale 0 and 0 / 0)
     } else if (SCALE == SCALE_TENSOR) {
         float amax = 0.f;
         for (int i = tid; i < n_aux; i += kThreads) amax = fmaxf(amax, aux[i]);
         amax = block_max<kNW>(amax, smem);
         s = scale_from_amax<DT, MODE>(amax);
+        fin = amax < __builtin_inff() && s > 0.f;  // (the fp8 floor rounds to 0 in fp16: an all-zero row has scale 0 and 0 / 0)
     } else {
         s = aux[0];
     }
@@ -67,10 +70,18 @@ __global__ __launch_bounds__(kThreads) void quant_rows_kernel(
     const float inv_s = 1.0f / s;
     constexpr bool F32Q = (SCALE == SCALE_STATIC);
     if (SCALE == SCALE_ROW && NC > 0) {
+        if (fin) {
 #pragma unroll
-        for (int c = 0; c < NC; c++) {
-            const int i = tid + c * kThreads;
-            if (i < nchunk) qr[i] = quant8<DT, MODE, Q_DT>(cache[c], s, inv_s);
+            for (int c = 0; c < NC; c++) {
+                const int i = tid + c * kThreads;
+                if (i < nchunk) qr[i] = quant8<DT, MODE, Q_DT, true>(cache[c], s, inv_s);
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < NC; c++) {
+                const int i = tid + c * kThreads;
+                if (i < nchunk) qr[i] = quant8<DT, MODE, Q_DT>(cache[c], s, inv_s);
+            }
         }
     } else if (F32Q) {
         if (static_f32) {
@@ -78,6 +89,8 @@ __global__ __launch_bounds__(kThreads) void quant_rows_kernel(
         } else {
             for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, MODE, Q_DIV_DT>(xr[i], s, inv_s);
         }
+    } else if (fin) {
+        for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, MODE, Q_DT, true>(xr[i], s, inv_s);
     } else {
         for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, MODE, Q_DT>(xr[i], s, inv_s);
     }
@@ -111,10 +124,18 @@ __global__ __launch_bounds__(kThreads) void quant_rows_wave_kernel(
         else ((uint16_t*)scale_out)[row] = Lo<DT>::from_f32(s);
     }
     const float inv_s = 1.0f / s;
+    if (amax < __builtin_inff() && s > 0.f) {  // wavefront-uniform: no quotient can be NaN
 #pragma unroll
-    for (int c = 0; c < NCW; c++) {
-        const int i = lane + c * kWave;
-        if (i < nchunk) qr[i] = quant8<DT, MODE, Q_DT>(cache[c], s, inv_s);
+        for (int c = 0; c < NCW; c++) {
+            const int i = lane + c * kWave;
+            if (i < nchunk) qr[i] = quant8<DT, MODE, Q_DT, true>(cache[c], s, inv_s);
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < NCW; c++) {
+            const int i = lane + c * kWave;
+            if (i < nchunk) qr[i] = quant8<DT, MODE, Q_DT>(cache[c], s, inv_s);
+        }
     }
 }
 
@@ -234,7 +255,13 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_quant_rows_kernel(
         else ((uint16_t*)scale_out)[row] = Lo<DT>::from_f32(s);
     }
     const float inv_s = 1.0f / s;
-    if (NC > 0) {
+    if (NC > 0 && amax < __builtin_inff() && s > 0.f) {  // block-uniform: no quotient can be NaN
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+            const int i = tid + c * kThreads;
+            if (i < nchunk) qr[i] = quant8<DT, QM, Q_DT, true>(cache[c], s, inv_s);
+        }
+    } else if (NC > 0) {
 #pragma unroll
         for (int c = 0; c < NC; c++) {
             const int i = tid + c * kThreads;
@@ -291,10 +318,18 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_quant_rows_wave_kernel(
         else ((uint16_t*)scale_out)[row] = Lo<DT>::from_f32(s);
     }
     const float inv_s = 1.0f / s;
+    if (amax < __builtin_inff() && s > 0.f) {  // wavefront-uniform: no quotient can be NaN
 #pragma unroll
-    for (int c = 0; c < NCW; c++) {
-        const int i = lane + c * kWave;
-        if (i < nchunk) qr[i] = quant8<DT, QM, Q_DT>(cache[c], s, inv_s);
+        for (int c = 0; c < NCW; c++) {
+            const int i = lane + c * kWave;
+            if (i < nchunk) qr[i] = quant8<DT, QM, Q_DT, true>(cache[c], s, inv_s);
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < NCW; c++) {
+            const int i = lane + c * kWave;
+            if (i < nchunk) qr[i] = quant8<DT, QM, Q_DT>(cache[c], s, inv_s);
+        }
     }
 }
 

@@ -48,7 +48,9 @@ __device__ __forceinline__ float quotient(float x, float s, float inv_s) {
     return Lo<DT>::round(x * inv_s);
 }
 
-template <int DT, int MODE, int QUOT>
+// FIN: the caller knows that no quotient can be NaN (the row's absmax is finite, so every element is finite, and the
+// scale is positive): the per-element NaN handling, which then never fires, is left out.
+template <int DT, int MODE, int QUOT, bool FIN = false>
 __device__ __forceinline__ uint2 quant8(uint4 raw, float s, float inv_s) {
     const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
     float f[8];
@@ -61,10 +63,10 @@ __device__ __forceinline__ uint2 quant8(uint4 raw, float s, float inv_s) {
     for (int i = 0; i < 8; i++) {
         float q = quotient<DT, QUOT>(f[i], s, inv_s);
         if (MODE == MODE_I8) {
-            f[i] = (q != q) ? 0.f : q;  // NaN narrows to 0 (what the reference's cast gives); clamp: see below
+            f[i] = (!FIN && q != q) ? 0.f : q;  // NaN narrows to 0 (what the reference's cast gives); clamp: see below
         } else {
             const float c = __builtin_amdgcn_fmed3f(q, QP<MODE>::lo, QP<MODE>::hi);
-            f[i] = (q != q) ? q : c;  // clamp keeps NaN, as torch.clamp does
+            f[i] = (!FIN && q != q) ? q : c;  // clamp keeps NaN, as torch.clamp does
         }
     }
     uint32_t out[2];
