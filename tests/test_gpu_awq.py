@@ -347,6 +347,45 @@ def test_decode_kernel_in_a_hip_graph(cuda, M, K, N):
     assert rel_err(out, ref) <= REL_TOL
 
 
+def test_decode_kernel_on_two_streams_at_once(cuda):
+    """Calls on different streams overlap on the GPU; each takes its own run of arrival tickets (the ring wraps
+    several times here), so every result must equal the one computed alone."""
+    from llmqrt_amd import _abi, workloads as W
+    L = _abi.lib()
+    K, N = 3584, 4608
+    qw, qz, s = (t.to(cuda) for t in W.awq_weights(N, K, 91))
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    Ms = (4, 48)
+    xs = [W.activations(M, K, 900 + i, dtype=torch.float16, outliers=False).to(cuda) for i, M in enumerate(Ms)]
+    nws = [L.llmq_awq_gemm_workspace_bytes(M, N, K) for M in Ms]
+    assert all(n > 0 for n in nws), "both shapes are meant to split K across blocks"
+    wsp = [torch.empty(n, dtype=torch.uint8, device=cuda) for n in nws]
+    alone = []
+    for i, M in enumerate(Ms):
+        out = torch.empty((M, N), dtype=torch.float16, device=cuda)
+        rc = L.llmq_awq_gemm(xs[i].data_ptr(), K, qw.data_ptr(), s.data_ptr(), qz.data_ptr(), None, out.data_ptr(), M, N, K,
+                             128, wsp[i].data_ptr(), nws[i], torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        alone.append(out)
+    reps = 300
+    outs = [[torch.empty((M, N), dtype=torch.float16, device=cuda) for _ in range(4)] for M in Ms]
+    torch.cuda.synchronize()
+    for r in range(reps):
+        for i, M in enumerate(Ms):
+            rc = L.llmq_awq_gemm(xs[i].data_ptr(), K, qw.data_ptr(), s.data_ptr(), qz.data_ptr(), None,
+                                 outs[i][r % 4].data_ptr(), M, N, K, 128, wsp[i].data_ptr(), nws[i], streams[i].cuda_stream)
+            assert rc == 0
+        if r % 4 == 3:
+            for st in streams:
+                st.synchronize()
+            for i in range(2):
+                for o in outs[i]:
+                    assert torch.equal(o, alone[i]), (r, i)
+                    o.zero_()
+    torch.cuda.synchronize()
+
+
 def test_decode_kernel_extreme_nibbles_and_zero_tokens(cuda, force_awq_plan):
     """All-15 weights against zero points 0 and all-0 weights against zero points 15 (the largest |q - z|), and a
     token block whose rows past M must not leak into the result."""
