@@ -407,25 +407,27 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     const float alpha = ep.alpha * (ep.alpha_dev ? *ep.alpha_dev : 1.0f);
     const bool out_vec = ((ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(out) & 15u) == 0);
     const bool raw_vec = (N & 3) == 0;
+    const bool plain = !ep.bias && alpha == 1.0f;  // block-uniform
 
     // Fast path (block-uniform): interior tile, fused epilogue, vector stores.  No per-element dtype
     // switches or bounds checks: ~5 VALU operations per output instead of several times that.
     if (!split && !acc_dump && out_vec && m0 + C::BM <= M && n0 + C::BN <= N &&
         (reinterpret_cast<uintptr_t>(ep.w_scale) & 15u) == 0) {
-        auto fast = [&](auto out_dt_c) {
+        auto fast = [&](auto out_dt_c, auto plain_c) {
             constexpr int ODT = decltype(out_dt_c)::value;
+            constexpr bool PLAIN = decltype(plain_c)::value;  // no bias term and alpha = 1: the scaled accumulator is the output
             // Wave tiles of 64 channels: transpose through LDS (8 KB per wavefront, 64 token rows at a time) so
             // that a store instruction writes 8 whole 128-byte rows instead of 32 pieces of 32 bytes.
-            constexpr bool LDS_EPI = LLMQ_LDS_EPILOGUE && C::TM % 2 == 0 && C::TN == 2 && C::LDS_BYTES >= (C::NT / kWave) * 8192u;
+            constexpr bool LDS_EPI = LLMQ_LDS_EPILOGUE && C::TM % 2 == 0 && C::TN % 2 == 0 && C::LDS_BYTES >= (C::NT / kWave) * 8192u;
             if constexpr (LDS_EPI) {
                 // Every scale and bias value is fetched before the first output store is issued: loads and stores
                 // share one wait counter, so a load issued after a store can only be waited for together with that
                 // store's completion (microseconds when every CU writes at once).
-                float sa_r[C::TM], sw_r[2][16], bb_r[2][16];
+                float sa_r[C::TM], sw_r[C::TN][16], bb_r[C::TN][16];
 #pragma unroll
                 for (int i = 0; i < C::TM; i++) sa_r[i] = ep.a_scale ? ep.a_scale[m0 + wm * C::WTM + i * 32 + l32] : 1.f;
 #pragma unroll
-                for (int j = 0; j < 2; j++)
+                for (int j = 0; j < C::TN; j++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
                         const int n = n0 + wn * C::WTN + j * 32 + 8 * g + 4 * khalf;
@@ -444,7 +446,10 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
 #pragma unroll
                 for (int p = 0; p < C::TM / 2; p++) {
 #pragma unroll
-                    for (int j = 0; j < 2; j++) {
+                  for (int jh = 0; jh < C::TN / 2; jh++) {  // 64 channels at a time
+#pragma unroll
+                    for (int jj = 0; jj < 2; jj++) {
+                        const int j = 2 * jh + jj;
 #pragma unroll
                         for (int ii = 0; ii < 2; ii++) {
                             const int i = 2 * p + ii;
@@ -457,7 +462,7 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
 #pragma unroll
                                 for (int e = 0; e < 4; e++) {
                                     const auto av = acc[i][j][4 * g + e];
-                                    h[e] = Lo<ODT>::from_f32(epi_value((float)av, sa, sw_r[j][4 * g + e], alpha, bb_r[j][4 * g + e]));
+                                    h[e] = Lo<ODT>::from_f32(epi_value<PLAIN>((float)av, sa, sw_r[j][4 * g + e], alpha, bb_r[j][4 * g + e]));
                                 }
                                 pk[g][0] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
                                 pk[g][1] = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
@@ -470,18 +475,19 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
                                     pk[2 * g][x] = sw2[0];
                                     pk[2 * g + 1][x] = sw2[1];
                                 }
-                                const int chunk = 4 * j + 2 * g + khalf;  // 8 channels = 16 bytes
+                                const int chunk = 4 * jj + 2 * g + khalf;  // 8 channels = 16 bytes
                                 region[row * 8 + (chunk ^ swz)] = make_uint4(pk[2 * g][0], pk[2 * g][1], pk[2 * g + 1][0], pk[2 * g + 1][1]);
                             }
                         }
                     }
-                    uint16_t* obase = reinterpret_cast<uint16_t*>(out) + (int64_t)(m0 + wm * C::WTM + p * 64) * ldo + n0 + wn * C::WTN;
+                    uint16_t* obase = reinterpret_cast<uint16_t*>(out) + (int64_t)(m0 + wm * C::WTM + p * 64) * ldo + n0 + wn * C::WTN + jh * 64;
 #pragma unroll
                     for (int it = 0; it < 8; it++) {
                         const int q = it * kWave + lane, row = q >> 3, c = q & 7;
                         const uint4 v = region[row * 8 + (c ^ ((row >> 1) & 7))];
                         store_streaming(obase + (int64_t)row * ldo + 8 * c, v);
                     }
+                  }
                 }
                 return;
             }
@@ -516,7 +522,7 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
                             const auto av = acc[i][j][4 * g + e];
-                            h[e] = Lo<ODT>::from_f32(epi_value((float)av, sa, sw[4 * g + e], alpha, bb[4 * g + e]));
+                            h[e] = Lo<ODT>::from_f32(epi_value<PLAIN>((float)av, sa, sw[4 * g + e], alpha, bb[4 * g + e]));
                         }
                         pk[g][0] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
                         pk[g][1] = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
@@ -535,8 +541,13 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
                 }
             }
         };
-        if (ep.out_dtype == LLMQ_BF16) fast(std::integral_constant<int, LLMQ_BF16>{});
-        else fast(std::integral_constant<int, LLMQ_F16>{});
+        if (plain) {
+            if (ep.out_dtype == LLMQ_BF16) fast(std::integral_constant<int, LLMQ_BF16>{}, std::true_type{});
+            else fast(std::integral_constant<int, LLMQ_F16>{}, std::true_type{});
+        } else {
+            if (ep.out_dtype == LLMQ_BF16) fast(std::integral_constant<int, LLMQ_BF16>{}, std::false_type{});
+            else fast(std::integral_constant<int, LLMQ_F16>{}, std::false_type{});
+        }
         return;
     }
 #pragma unroll
@@ -588,7 +599,7 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const auto av = acc[i][j][4 * g + e];
-                    h[e] = to_out(epi_value((float)av, sa, sw[4 * g + e], alpha, bb[4 * g + e]), ep.out_dtype);
+                    h[e] = to_out(plain ? epi_value<true>((float)av, sa, sw[4 * g + e], alpha, 0.f) : epi_value<false>((float)av, sa, sw[4 * g + e], alpha, bb[4 * g + e]), ep.out_dtype);
                 }
                 pk[g][0] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
                 pk[g][1] = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
@@ -647,7 +658,7 @@ __global__ __launch_bounds__(256) void splitk_epilogue_kernel(const void* __rest
         }
         const float sa = ep.a_scale ? ep.a_scale[m] : 1.f, sw = ep.w_scale ? ep.w_scale[n] : 1.f;
         const float bb = ep.bias ? ep.beta * load_as_f32(ep.bias, ep.bias_dtype, n) : 0.f;
-        reinterpret_cast<uint16_t*>(out)[(int64_t)m * ldo + n] = to_out(epi_value(accf, sa, sw, alpha, bb), ep.out_dtype);
+        reinterpret_cast<uint16_t*>(out)[(int64_t)m * ldo + n] = to_out((!ep.bias && alpha == 1.0f) ? epi_value<true>(accf, sa, sw, alpha, 0.f) : epi_value<false>(accf, sa, sw, alpha, bb), ep.out_dtype);
     }
 }
 
@@ -690,8 +701,8 @@ template <bool FP8, int AFMT, bool DMA>
 int launch_shape(const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb, int M, int N, int K, const Plan& p,
                  const Epilogue& ep, void* out, int64_t ldo, void* acc_dump, void* ws, hipStream_t st) {
     switch (p.cfg) {
-        case 0: return launch_cfg<GemmCfg<256, 256, 64, 2, 2, FP8, AFMT, 2, DMA && !FP8>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
         case 1: return launch_cfg<GemmCfg<256, 256, 64, 2, 4, FP8, AFMT, 2, DMA && !FP8>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
+        case 0: return launch_cfg<GemmCfg<256, 256, 64, 2, 2, FP8, AFMT, 2, DMA && !FP8>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
         case 2: return launch_cfg<GemmCfg<256, 128, 64, 2, 2, FP8, AFMT, 2, DMA && !FP8>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
         case 3: return launch_cfg<GemmCfg<128, 128, 64, 2, 2, FP8, AFMT, 2, DMA && !FP8>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);
         case 4: return launch_cfg<GemmCfg<64, 128, 128, 2, 2, FP8, AFMT, 2, DMA>>(A, lda, B, ldb, M, N, K, p, ep, out, ldo, acc_dump, ws, st);

@@ -29,9 +29,12 @@ template <> struct Lo<LLMQ_F16> {
 // the bias term.  The result is made opaque to the compiler before it is converted to the output type: otherwise
 // the fma and a conversion to fp16 may or may not be merged into one mixed-precision instruction that rounds the
 // exact sum straight to fp16, and two code paths could disagree on ties of the double rounding.
+// PLAIN (no bias term and alpha = 1): the scaled accumulator is the result, as in the reference's epilogue without a bias.
+template <bool PLAIN = false>
 __device__ __forceinline__ float epi_value(float acc, float sa, float sw, float alpha, float bb) {
     float p = (acc * sa) * sw;
     asm volatile("" : "+v"(p));  // the scaled accumulator is a value of its own: never contracted into what follows
+    if constexpr (PLAIN) return p;
     float r = fmaf(alpha, p, bb);
     asm volatile("" : "+v"(r));
     return r;
