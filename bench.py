@@ -316,7 +316,7 @@ def details_awq(dev, full=True):
             x = W.activations(M, K, W.seed_for(3, 10 * pi + mi), dtype=torch.float16, outliers=False).to(dev)
             out = torch.empty((M, N), dtype=torch.float16, device=dev)
             wsb = L.llmq_awq_gemm_workspace_bytes(M, N, K)
-            wsp = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+            wsp = torch.zeros(max(wsb, 16), dtype=torch.uint8, device=dev)  # arrival counters at its start: cleared once
 
             def mk(c):
                 def f():
@@ -399,7 +399,7 @@ def awq_only(dev, steps, warmup):
         for mi, M in enumerate(W.AWQ_M):
             x = W.activations(M, K, W.seed_for(3, 10 * pi + mi), dtype=torch.float16, outliers=False).to(dev)
             out = torch.empty((M, N), dtype=torch.float16, device=dev)
-            wsp = torch.empty(max(L.llmq_awq_gemm_workspace_bytes(M, N, K), 16), dtype=torch.uint8, device=dev)
+            wsp = torch.zeros(max(L.llmq_awq_gemm_workspace_bytes(M, N, K), 16), dtype=torch.uint8, device=dev)
             launches.append((x, out, wsp, copies, M, N, K))
             order.append(f"{pname}_M{M}")
     torch.cuda.synchronize()
@@ -432,7 +432,7 @@ def awq_prefill_only(dev, steps, warmup):
         for mi, M in enumerate(AWQ_PREFILL_M):
             x = W.activations(M, K, W.seed_for(3, 50 * pi + mi), dtype=torch.float16, outliers=False).to(dev)
             out = torch.empty((M, N), dtype=torch.float16, device=dev)
-            wsp = torch.empty(max(L.llmq_awq_gemm_workspace_bytes(M, N, K), 16), dtype=torch.uint8, device=dev)
+            wsp = torch.zeros(max(L.llmq_awq_gemm_workspace_bytes(M, N, K), 16), dtype=torch.uint8, device=dev)
             launches.append((x, out, wsp, (qw, qz, sc), M, N, K))
             order.append(f"{pname}_M{M}")
     torch.cuda.synchronize()

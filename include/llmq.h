@@ -63,6 +63,18 @@ int llmq_quant_i8_per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, i
                              int8_t* q, void* scale, int scale_dtype,
                              void* workspace, size_t workspace_bytes, llmq_stream_t stream);
 
+/* The same two quantizers with the lower clamp bound of the absmax given by the caller instead of 1e-5:
+ * absmax_floor = 1e-8 replaces dynamic_quantize_activation_per_token_absmax and
+ * dynamic_quantize_activation_per_tensor_absmax, utils/quantization_utils.py:57-71 (which also overwrite
+ * their input with the rounded quotients; x is left untouched here).  The bound is rounded to x_dtype
+ * like every other value of the chain (1e-8 is 0 in fp16).  absmax_floor >= 0. */
+int llmq_quant_i8_per_token_floor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                  int8_t* q, void* scale, int scale_dtype, float absmax_floor,
+                                  llmq_stream_t stream);
+int llmq_quant_i8_per_tensor_floor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                   int8_t* q, void* scale, int scale_dtype, float absmax_floor,
+                                   void* workspace, size_t workspace_bytes, llmq_stream_t stream);
+
 /* Replaces per_token_quantize, nn_models/modules/linear/linear_fp8.py:40-63.
  * q: e4m3fn bytes [M, K] contiguous; scale: fp32 [M]. */
 int llmq_quant_fp8_per_token(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
@@ -161,6 +173,22 @@ int llmq_gemm_fp8(const uint8_t* A, int a_format, int64_t lda, const uint8_t* B,
 
 size_t llmq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
+/* llmq_gemm_fp8 with the output quantization of FP8StaticLinear.forward folded into the epilogue
+ * (nn_models/modules/linear/linear_fp8.py:309-311: static_per_tensor_quantize(output, output_scale), then
+ * qoutput.to(dtype) * output_scale): the GEMM result is rounded to inter_dtype (bf16 / f16, the module's dtype),
+ * divided by *out_scale in fp32, clamped to +-448, rounded to e4m3fn, widened again and multiplied by *out_scale.
+ * out: fp32 [M, N] (the reference's product of a 16-bit tensor and a one-element fp32 tensor is fp32), row stride
+ * ldo elements.  out_scale: fp32 device scalar.  One launch instead of three and no extra trips of the [M, N] output
+ * through HBM.  workspace: >= llmq_gemm_fp8_quantized_output_workspace_bytes(M, N, K). */
+int llmq_gemm_fp8_quantized_output(const uint8_t* A, int a_format, int64_t lda, const uint8_t* B, int64_t ldb,
+                                   const float* a_scale, const float* w_scale,
+                                   float alpha, const float* alpha_dev,
+                                   const void* bias, int bias_dtype, float beta,
+                                   const float* out_scale, float* out, int inter_dtype, int64_t ldo,
+                                   int64_t M, int64_t N, int64_t K,
+                                   void* workspace, size_t workspace_bytes, llmq_stream_t stream);
+size_t llmq_gemm_fp8_quantized_output_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
 /* llmq_gemm_w8a8 for callers that cannot allocate or pass a workspace: code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments and
  * results as llmq_gemm_w8a8 without acc_dump / workspace: the split-K partial sums go to a static device array
@@ -207,13 +235,13 @@ int llmq_linear_fp8_dynamic(const void* x, int x_dtype, int64_t ldx, const uint8
                             int64_t K, uint8_t* q_dump, float* scale_dump, float* acc_dump, llmq_stream_t stream);
 int llmq_linear_dynamic_max_tokens(int64_t K);
 /* Tuning / test hook: 0 = two 16-channel tiles per wavefront x 4 wavefronts per block, 1 = one tile x 8 wavefronts,
- * -1 = built-in choice.  Process-global, not thread-safe. */
+ * -1 = built-in choice.  Per host thread (thread-local state): it affects only calls made later by the thread that set it. */
 int llmq_linear_dynamic_force_variant(int v);
 
 /* Tuning / test hook with no counterpart in the reference: force tile configuration `cfg`
  * (0 .. llmq_gemm_num_configs()-1) and K split `splits` for every later GEMM call of this
  * process; cfg < 0 restores the built-in heuristic.  cfg | 64 keeps the register-staged main loop,
- * 100 .. 105 pick a variant of the few-token kernel.  Process-global, not thread-safe. */
+ * 100 .. 105 pick a variant of the few-token kernel.  Per host thread (thread-local state): it affects only calls made later by the thread that set it. */
 int llmq_gemm_force_plan(int cfg, int splits);
 int llmq_gemm_num_configs(void);
 
@@ -232,13 +260,23 @@ int llmq_gemm_num_configs(void);
  * unrounded, exact (q - z) * s in fp32, instead of rounded to fp16 first); above 64 tokens
  * an fp16 tile GEMM dequantizes the weights on their way into LDS.  All are within 1e-2 of the
  * dequantize-then-matmul math.
- * workspace: >= llmq_awq_gemm_workspace_bytes(M,N,K) bytes, 16-byte aligned, contents irrelevant. */
+ * workspace: >= llmq_awq_gemm_workspace_bytes(M,N,K) bytes, 16-byte aligned.  Its first
+ * llmq_awq_workspace_ticket_bytes() bytes are the arrival counters of the few-token kernel's K split:
+ * they must be zero when a call starts and every call leaves them zero, so a workspace is cleared once
+ * (llmq_awq_workspace_init, or any zero fill) when it is allocated and can then serve any sequence of calls
+ * of any shape; the contents of the rest are irrelevant.  Calls that may overlap in time (different
+ * streams, a captured launch replayed beside eager calls) need different workspaces. */
 int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight, const void* scales,
                   const int32_t* qzeros, const void* bias, void* out,
                   int64_t M, int64_t N, int64_t K, int64_t group,
                   void* workspace, size_t workspace_bytes, llmq_stream_t stream);
 
 size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/* No counterpart in the reference (its split-K ends in fp16 atomics on the output, awq_kernels.py:253-267):
+ * size of the counter area at the start of an AWQ workspace, and a launch on `stream` that zeroes it. */
+size_t llmq_awq_workspace_ticket_bytes(void);
+int llmq_awq_workspace_init(void* workspace, size_t workspace_bytes, llmq_stream_t stream);
 
 /* Tuning / test hook with no counterpart in the reference: force the kernel variant of
  * llmq_awq_gemm for every later call of this process: v = 1 or 2 words per lane of the streaming
@@ -248,7 +286,7 @@ size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * (0 = heuristic); the wavefronts per block along K of the streaming kernel (4 or 8), or the K slices
  * inside a block of the few-token kernel (1, 2 or 4, v = 8 only); 0 = heuristic.
  * v + 32 keeps the tile kernel's register-staged activation loads (default: straight into LDS when K % 64 == 0).
- * Process-global, not thread-safe. */
+ * Per host thread (thread-local state): it affects only calls made later by the thread that set it. */
 int llmq_awq_force_plan(int v, int splits, int k_waves);
 
 /* out: fp16 [K, N] contiguous = fp16(q - z) * s, bit-exact with

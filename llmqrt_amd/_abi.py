@@ -27,6 +27,8 @@ SIGNATURES = {
     "llmq_quant_i8_per_token": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _int, _vp]),
     "llmq_quant_i8_weight_per_channel": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "llmq_quant_i8_per_tensor": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _int, _vp, _sz, _vp]),
+    "llmq_quant_i8_per_token_floor": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _int, _f32, _vp]),
+    "llmq_quant_i8_per_tensor_floor": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _int, _f32, _vp, _sz, _vp]),
     "llmq_quant_fp8_per_token": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp]),
     "llmq_quant_fp8_per_tensor": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
     "llmq_quant_fp8_static": (_int, [_vp, _int, _i64, _i64, _i64, _vp, _vp, _int, _vp]),
@@ -48,11 +50,16 @@ SIGNATURES = {
     "llmq_linear_fp8_dynamic": (_int, [_vp, _int, _i64, _vp, _i64, _vp, _vp, _int, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
     "llmq_linear_dynamic_max_tokens": (_int, [_i64]),
     "llmq_linear_dynamic_force_variant": (_int, [_int]),
+    "llmq_gemm_fp8_quantized_output": (_int, [_vp, _int, _i64, _vp, _i64, _vp, _vp, _f32, _vp, _vp, _int, _f32, _vp, _vp, _int,
+                                              _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
+    "llmq_gemm_fp8_quantized_output_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "llmq_gemm_force_plan": (_int, [_int, _int]),
     "llmq_gemm_num_configs": (_int, []),
     "llmq_awq_gemm": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
     "llmq_awq_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "llmq_awq_force_plan": (_int, [_int, _int, _int]),
+    "llmq_awq_workspace_ticket_bytes": (_sz, []),
+    "llmq_awq_workspace_init": (_int, [_vp, _sz, _vp]),
     "llmq_awq_dequant": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "llmq_awq_dequant_t": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
 }
@@ -102,10 +109,13 @@ def stream_of(t: torch.Tensor) -> int:
 
 
 class _Workspaces:
-    """One grow-only scratch tensor per (device, stream): the C library never allocates."""
+    """One grow-only scratch tensor per (device, stream): the C library never allocates.
+    zeroed: every new buffer starts as zeros (the AWQ workspace begins with arrival counters that must be zero before
+    the first call and that every call leaves zero)."""
 
-    def __init__(self):
+    def __init__(self, zeroed: bool = False):
         self._buf = {}
+        self._zeroed = zeroed
 
     def get(self, device: torch.device, nbytes: int) -> torch.Tensor | None:
         if nbytes == 0:
@@ -113,9 +123,11 @@ class _Workspaces:
         key = (device.index, torch.cuda.current_stream(device).cuda_stream)
         buf = self._buf.get(key)
         if buf is None or buf.numel() < nbytes:
-            buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+            alloc = torch.zeros if self._zeroed else torch.empty
+            buf = alloc(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
             self._buf[key] = buf
         return buf
 
 
 workspaces = _Workspaces()
+awq_workspaces = _Workspaces(zeroed=True)  # never shared with another op: their partial sums would overwrite the counters

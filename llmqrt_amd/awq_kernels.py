@@ -97,7 +97,7 @@ def awq_gemm_triton(input: torch.Tensor, qweight: torch.Tensor, scales: torch.Te
         x = x.contiguous()
     result = torch.empty((M, N), dtype=scales.dtype, device=input.device)
     L = _abi.lib()
-    ws = _abi.workspaces.get(x.device, L.llmq_awq_gemm_workspace_bytes(M, N, K))
+    ws = _abi.awq_workspaces.get(x.device, L.llmq_awq_gemm_workspace_bytes(M, N, K))
     _abi.check(L.llmq_awq_gemm(x.data_ptr(), x.stride(0), qweight.data_ptr(), scales.data_ptr(), qzeros.data_ptr(),
                                _abi.ptr(bias), result.data_ptr(), M, N, K, group_size, _abi.ptr(ws),
                                ws.numel() if ws is not None else 0, _abi.stream_of(x)), "llmq_awq_gemm")

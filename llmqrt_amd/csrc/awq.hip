@@ -678,7 +678,7 @@ struct AwqPlan { int v, mt, splits, chunks_per_block; };
 
 inline int cdiv(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
-int g_force_v = 0, g_force_splits = 0, g_force_kw = 0;  // tuning hook (llmq_awq_force_plan)
+thread_local int g_force_v = 0, g_force_splits = 0, g_force_kw = 0;  // tuning hook (llmq_awq_force_plan): per host thread
 
 // Generic kernel (any group size, up to 64 tokens): 4 wavefronts split the block's K range.
 AwqPlan make_awq_plan(int64_t M, int64_t N, int64_t K) {
@@ -768,8 +768,11 @@ using namespace llmq;
 extern "C" int llmq_awq_force_plan(int v, int splits, int k_waves) {
     const int staged = v >= 0 ? (v & 32) : 0;  // + 32: the tile kernel keeps its register-staged activation loads
     if (v >= 0) v &= ~32;
-    set_awq_tile_direct_loads(staged ? 0 : 1);
-    if (v < 0 || v > 11 || splits < 0 || splits > 64 || (k_waves != 0 && k_waves != 1 && k_waves != 2 && k_waves != 4 && k_waves != 8)) return LLMQ_ERR_SHAPE;
+    if (v < 0 || v > 11 || splits < 0 || splits > 64) return LLMQ_ERR_SHAPE;
+    // K slices of the few-token kernel: 1, 2, 4 (v = 0 or 8 .. 11); wavefronts along K of the streaming kernel: 4, 8
+    const bool few = v == 0 || v >= 8;
+    if (k_waves != 0 && !(k_waves == 4 || (few && (k_waves == 1 || k_waves == 2)) || (!few && k_waves == 8))) return LLMQ_ERR_SHAPE;
+    set_awq_tile_direct_loads(staged ? 0 : 1);  // state changes only once the arguments are accepted
     g_force_v = v;
     g_force_splits = splits;
     g_force_kw = k_waves;
@@ -798,7 +801,15 @@ extern "C" size_t llmq_awq_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K)
         }
         if (need > total) total = need;
     }
-    return total;
+    return total ? kAwqTicketBytes + total : 0;  // the arrival counters come first
+}
+
+extern "C" size_t llmq_awq_workspace_ticket_bytes(void) { return kAwqTicketBytes; }
+
+extern "C" int llmq_awq_workspace_init(void* workspace, size_t workspace_bytes, llmq_stream_t stream) {
+    if (!workspace || workspace_bytes == 0) return LLMQ_OK;
+    if (reinterpret_cast<uintptr_t>(workspace) & 15u) return LLMQ_ERR_ALIGN;
+    return awq_clear_tickets(workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight, const void* scales,
@@ -814,7 +825,10 @@ extern "C" int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight,
         (reinterpret_cast<uintptr_t>(qzeros) & 15u) || (reinterpret_cast<uintptr_t>(workspace) & 15u))
         return LLMQ_ERR_ALIGN;
     hipStream_t st = (hipStream_t)stream;
-    float* ws = (float*)workspace;
+    // workspace = arrival counters (kAwqTicketBytes, zero between calls), then partial sums (contents irrelevant)
+    unsigned int* tickets = workspace_bytes > kAwqTicketBytes ? (unsigned int*)workspace : nullptr;
+    float* ws = tickets ? (float*)((unsigned char*)workspace + kAwqTicketBytes) : nullptr;
+    workspace_bytes = tickets ? workspace_bytes - kAwqTicketBytes : 0;
     const uint32_t* qw = (const uint32_t*)qweight;
     const uint32_t* qz = (const uint32_t*)qzeros;
     const uint16_t* sc = (const uint16_t*)scales;
@@ -837,7 +851,7 @@ extern "C" int llmq_awq_gemm(const void* x, int64_t ldx, const int32_t* qweight,
     if (decode16_path(M, N, K, group)) {
         const AwqDecodePlan d = decode16_plan(M, N, K);
         if (d.splits > 1 && (!ws || workspace_bytes < awq_decode_workspace_bytes(d, M, N))) return LLMQ_ERR_WORKSPACE;
-        return launch_awq_decode(d, (const uint16_t*)x, ldx, qw, sc, qz, bs, (uint16_t*)out, ws, (int)M, Ni, Ki, st);
+        return launch_awq_decode(d, (const uint16_t*)x, ldx, qw, sc, qz, bs, (uint16_t*)out, tickets, ws, (int)M, Ni, Ki, st);
     }
     // tokens are processed in slabs of at most 64 rows (4 MFMA token tiles per weight pass)
     for (int64_t m0 = 0; m0 < M; m0 += 64) {

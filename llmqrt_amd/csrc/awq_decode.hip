@@ -19,10 +19,9 @@
 //     (0.75 VALU operations per weight plus 64 per group and wavefront.)
 //   * A K split across blocks writes fp32 partial sums [split][M][N] to the caller's workspace; the block that
 //     arrives last at a column tile adds them in split order and writes the output: one launch, results
-//     independent of scheduling.  Arrivals are counted in a ring of self-resetting tickets that the library owns
-//     (a zero-initialised static device array; every call takes fresh slots, so concurrent calls do not share any).
+//     independent of scheduling.  Arrivals are counted in self-resetting tickets at the start of that workspace
+//     (cleared once by its owner; calls that may overlap in time use different workspaces).
 #include <algorithm>
-#include <atomic>
 #include <type_traits>
 
 #include "awq_plans.h"
@@ -54,7 +53,6 @@ __host__ __device__ constexpr int rev_nibble_d(int j) { return ((j & 1) << 2) | 
 // Tickets of neighbouring tiles are 256 bytes apart so that their atomics land in different memory channels
 // (adjacent words were measured 1-3 us slower per launch).
 constexpr int kTicketStride = 64;  // in 4-byte words
-constexpr int kTicketRing = 1 << 18;  // words in the ring of tickets
 template <int TILE_CH, int NT>
 __device__ __forceinline__ void finish_split_tile(const float* ptile, int M, int N, int tile, int ks, int splits,
                                                   float* partials, int64_t plane, unsigned int* tickets,
@@ -377,9 +375,9 @@ inline int cdiv_d(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 }  // namespace
 
 bool awq_decode_supported(int64_t M, int64_t N, int64_t K, int64_t group) {
-    // a call's tickets (one per column tile and token slab) must fit in half of the ring
+    // a call's tickets (one per column tile and token slab) must fit in the ticket area of the workspace
     return M >= 1 && M <= 64 && group == kGroup && (N % 32) == 0 && (K % kGroup) == 0 &&
-           2 * ((M + 15) / 16) * (N / 256 + 1) <= kTicketRing / kTicketStride;
+           (size_t)((M + 15) / 16) * (N / 256 + 1) * kTicketStride * sizeof(unsigned int) <= kAwqTicketBytes;
 }
 
 // Column tile width (CS wavefronts = 16*CS words), prefetch depth, K slices per block and K split.  Measured on the
@@ -442,44 +440,29 @@ size_t awq_decode_workspace_bytes(const AwqDecodePlan& p, int64_t M, int64_t N) 
     return p.splits > 1 ? (size_t)p.splits * M * N * sizeof(float) : 0;
 }
 
-// Arrival tickets: a ring of counters, all zero between calls (each returns to zero with its last arrival).  A call
-// reserves a run of consecutive slots at a cursor that only moves forward; a reservation that would cross the end of
-// the ring is dropped and taken again (the next one starts near the front and cannot cross: a run is at most half
-// the ring), so no two reservations ever overlap until the cursor has gone once around, i.e. two calls can only meet
-// on a slot if more than kTicketRing / run later calls were issued while the first had still not run.  One copy per GPU.
-static __device__ unsigned int g_ticket_ring[kTicketRing];
-static unsigned int* g_ticket_ptr[64] = {};  // device address of each GPU's copy, looked up once per device
+// Arrival tickets: one counter per column tile and token slab, kTicketStride words apart, at the start of the caller's
+// workspace (kAwqTicketBytes).  They must be zero when a call starts and are zero again when it ends (each returns to
+// zero with its last arrival), so a workspace is cleared once, when it is allocated, and calls that may overlap in
+// time use different workspaces, exactly as for the partial sums behind them.  The library keeps no state of its own.
+__global__ void awq_clear_tickets_kernel(unsigned int* p, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0u;
+}
 
-static int ticket_slots(int tiles_n, unsigned int** out) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LLMQ_ERR_LAUNCH;
-    if (!g_ticket_ptr[dev]) {
-        void* p = nullptr;
-        if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_ticket_ring)) != hipSuccess || !p) return LLMQ_ERR_LAUNCH;
-        g_ticket_ptr[dev] = static_cast<unsigned int*>(p);  // benign if two threads race: same address
-    }
-    static std::atomic<unsigned long long> cursor{0};
-    const unsigned long long run = (unsigned long long)tiles_n * kTicketStride;
-    if (2 * run > kTicketRing) return LLMQ_ERR_SHAPE;  // awq_decode_supported keeps callers below this
-    unsigned long long at;
-    do {
-        at = cursor.fetch_add(run, std::memory_order_relaxed) % kTicketRing;
-    } while (at + run > kTicketRing);
-    *out = g_ticket_ptr[dev] + at;
-    return LLMQ_OK;
+int awq_clear_tickets(void* workspace, size_t bytes, hipStream_t st) {
+    const size_t n = (bytes < kAwqTicketBytes ? bytes : kAwqTicketBytes) / sizeof(unsigned int);
+    if (n == 0) return LLMQ_OK;
+    hipLaunchKernelGGL(awq_clear_tickets_kernel, dim3(64), dim3(256), 0, st, static_cast<unsigned int*>(workspace), n);
+    return launch_status();
 }
 
 int launch_awq_decode(const AwqDecodePlan& p, const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales,
-                      const uint32_t* qz, const uint16_t* bias, uint16_t* out, float* ws, int M, int N, int K,
-                      hipStream_t st) {
+                      const uint32_t* qz, const uint16_t* bias, uint16_t* out, unsigned int* tickets, float* ws, int M,
+                      int N, int K, hipStream_t st) {
     const int tiles_n = cdiv_d(N / 8, 16 * p.cs);
     const int slabs = cdiv_d(M, 16), work = tiles_n * p.splits;
     const dim3 grid((unsigned)(slabs == 1 ? work : cdiv_d(work, 8) * 8 * slabs));
-    unsigned int* tickets = nullptr;
-    if (p.splits > 1) {
-        const int rc = ticket_slots(tiles_n * slabs, &tickets);
-        if (rc != LLMQ_OK) return rc;
-    }
+    if (p.splits > 1 && (!tickets || (size_t)tiles_n * slabs * kTicketStride * sizeof(unsigned int) > kAwqTicketBytes))
+        return LLMQ_ERR_WORKSPACE;
 #define LLMQ_DECODE_RM(CS_, PD_, RM_, KS_)                                                                            \
     hipLaunchKernelGGL((awq_decode_kernel<CS_, PD_, RM_, KS_>), grid, dim3(CS_ * KS_ * kWave), 0, st, x, ldx, qw, scales, \
                        qz, bias, out, ws, tickets, M, N, K, p.groups_per_block, tiles_n, p.splits, slabs)

@@ -349,7 +349,7 @@ int launch_tile_impl(const uint16_t* x, int64_t ldx, const uint32_t* qw, const u
     return launch_status();
 }
 
-int g_awq_tile_dma = 1;  // 0 keeps the register-staged activation loads (tuning / test hook)
+thread_local int g_awq_tile_dma = 1;  // 0 keeps the register-staged activation loads (tuning / test hook, per host thread)
 
 template <class C>
 int launch_tile(const uint16_t* x, int64_t ldx, const uint32_t* qw, const uint16_t* scales, const uint32_t* qz,

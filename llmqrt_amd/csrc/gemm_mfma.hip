@@ -26,7 +26,7 @@ int launch_gemm_skinny(bool fp8, int a_format, int t, int nw, const uint8_t* A, 
 namespace {
 
 // Tuning/diagnostic knob (llmq_gemm_force_plan): forces a tile configuration and K split.
-int g_force_cfg = -1, g_force_splits = 1, g_force_dma = -1;  // g_force_dma: 0 = register-staged loop only
+thread_local int g_force_cfg = -1, g_force_splits = 1, g_force_dma = -1;  // per host thread; g_force_dma: 0 = register-staged loop only
 bool plan_override(int& cfg, int& splits) {
     if (g_force_cfg < 0) return false;
     cfg = g_force_cfg;
@@ -137,10 +137,12 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, double mfma_scale = 1.0, bool fp
 }
 
 // op: 0 int8, 1 fp8 (a_format picks the A format), 2 fp16 (K, lda, ldb in bytes, i.e. twice the element counts)
+// out_scale (device scalar, may be null): out is fp32 [M, N] holding the out_dtype result after a round trip through
+// e4m3fn on that scale (tile kernel's general epilogue; no few-token kernel, no tail split)
 int gemm_entry(int op, int a_format, const uint8_t* A, int64_t lda, const uint8_t* B, int64_t ldb,
                const float* a_scale, const float* w_scale, float alpha, const float* alpha_dev, const void* bias,
                int bias_dtype, float beta, void* out, int out_dtype, int64_t ldo, int64_t M, int64_t N, int64_t K,
-               void* acc_dump, void* ws, size_t ws_bytes, hipStream_t st) {
+               void* acc_dump, void* ws, size_t ws_bytes, hipStream_t st, const float* out_scale = nullptr) {
     const bool fp8 = op == 1;
     if (M < 0 || N < 0 || K < 0) return LLMQ_ERR_SHAPE;
     if (M == 0 || N == 0) return LLMQ_OK;
@@ -152,7 +154,7 @@ int gemm_entry(int op, int a_format, const uint8_t* A, int64_t lda, const uint8_
     if (fp8 && a_format != LLMQ_E4M3 && a_format != LLMQ_E5M2) return LLMQ_ERR_DTYPE;
     if (!aligned16(A) || !aligned16(B)) return LLMQ_ERR_ALIGN;
     int sk_t, sk_nw;
-    if (op != 2 && skinny_plan(M, N, K, sk_t, sk_nw)) {
+    if (op != 2 && !out_scale && skinny_plan(M, N, K, sk_t, sk_nw)) {
         const SkinnyEpilogue sep{a_scale, w_scale, alpha_dev, bias, alpha, beta, bias_dtype, out_dtype};
         return launch_gemm_skinny(fp8, a_format == LLMQ_E5M2 ? 1 : 0, sk_t, sk_nw, A, lda, B, ldb, (int)M, (int)N, (int)K, sep,
                                   out, ldo, acc_dump, st);
@@ -166,7 +168,7 @@ int gemm_entry(int op, int a_format, const uint8_t* A, int64_t lda, const uint8_
         if (!ws || ws_bytes < (size_t)p.splits * M * N * 4) return LLMQ_ERR_WORKSPACE;
     }
     auto run = [&](const Plan& pl, const uint8_t* Bp, const float* wsc, const void* bs, void* o, int64_t n) {
-        Epilogue ep{a_scale, wsc, alpha_dev, bs, alpha, beta, bias_dtype, out_dtype};
+        Epilogue ep{a_scale, wsc, alpha_dev, bs, alpha, beta, bias_dtype, out_dtype, out_scale};
         const bool dma = g_force_dma != 0;
         if (op == 2) return launch_gemm_f16(A, lda, Bp, ldb, (int)M, (int)n, (int)K, pl, ep, o, ldo, acc_dump, ws, dma, st);
         if (!fp8) return launch_gemm_i8(A, lda, Bp, ldb, (int)M, (int)n, (int)K, pl, ep, o, ldo, acc_dump, ws, dma, st);
@@ -178,7 +180,7 @@ int gemm_entry(int op, int a_format, const uint8_t* A, int64_t lda, const uint8_
     // whole number of rounds: the first part keeps the big tiles and ends with every CU busy, the rest runs as one
     // round of 128x256 tiles (twice the blocks, half the time each).  Measured: 8192 x 4608 x 3584 (2.25 rounds)
     // and 8192 x 37888 x 3584 (18.5 rounds).
-    if (g_force_cfg < 0 && p.cfg == 6 && p.splits == 1 && !acc_dump && K % 128 == 0) {
+    if (g_force_cfg < 0 && p.cfg == 6 && p.splits == 1 && !acc_dump && !out_scale && K % 128 == 0) {
         const int64_t tm = cdiv(M, 256), tn = cdiv(N, 256), tiles = tm * tn, tail = tiles % kNumCu, full = tiles - tail;
         if (full >= kNumCu && tail > 0 && tail <= 160 && full % tm == 0) {
             const int64_t n1 = full / tm * 256, n2 = N - n1;
@@ -276,6 +278,24 @@ extern "C" int llmq_gemm_fp8(const uint8_t* A, int a_format, int64_t lda, const 
                              size_t workspace_bytes, llmq_stream_t stream) {
     return gemm_entry(1, a_format, A, lda, B, ldb, a_scale, w_scale, alpha, alpha_dev, bias, bias_dtype, beta, out,
                       out_dtype, ldo, M, N, K, acc_dump, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int llmq_gemm_fp8_quantized_output(const uint8_t* A, int a_format, int64_t lda, const uint8_t* B, int64_t ldb,
+                                              const float* a_scale, const float* w_scale, float alpha,
+                                              const float* alpha_dev, const void* bias, int bias_dtype, float beta,
+                                              const float* out_scale, float* out, int inter_dtype, int64_t ldo, int64_t M,
+                                              int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                                              llmq_stream_t stream) {
+    if (!out_scale) return LLMQ_ERR_NULL;
+    // the few-token kernel is not used here: size the workspace for the tile kernel's plan
+    return gemm_entry(1, a_format, A, lda, B, ldb, a_scale, w_scale, alpha, alpha_dev, bias, bias_dtype, beta, out,
+                      inter_dtype, ldo, M, N, K, nullptr, workspace, workspace_bytes, (hipStream_t)stream, out_scale);
+}
+
+extern "C" size_t llmq_gemm_fp8_quantized_output_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    const Plan p = make_plan(M, N, K, 1.0, true);
+    return p.splits > 1 ? (size_t)p.splits * M * N * 4 : 0;
 }
 
 extern "C" size_t llmq_gemm_f16_workspace_bytes(int64_t M, int64_t N, int64_t K) {

@@ -16,6 +16,8 @@ struct Epilogue {
     const void* bias;       // [N] or null
     float alpha, beta;
     int bias_dtype, out_dtype;
+    const float* out_scale;  // device scalar or null.  Set: the value rounded to out_dtype makes a round trip through
+                             // e4m3fn on this scale and `out` is fp32 [M, N] (FP8 static linear with quantize_output)
 };
 
 struct Plan {

@@ -408,10 +408,11 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
     const bool out_vec = ((ldo & 7) == 0) && ((reinterpret_cast<uintptr_t>(out) & 15u) == 0);
     const bool raw_vec = (N & 3) == 0;
     const bool plain = !ep.bias && alpha == 1.0f;  // block-uniform
+    const float out_scale = ep.out_scale ? *ep.out_scale : 1.0f;
 
     // Fast path (block-uniform): interior tile, fused epilogue, vector stores.  No per-element dtype
     // switches or bounds checks: ~5 VALU operations per output instead of several times that.
-    if (!split && !acc_dump && out_vec && m0 + C::BM <= M && n0 + C::BN <= N &&
+    if (!split && !acc_dump && !ep.out_scale && out_vec && m0 + C::BM <= M && n0 + C::BN <= N &&
         (reinterpret_cast<uintptr_t>(ep.w_scale) & 15u) == 0) {
         auto fast = [&](auto out_dt_c, auto plain_c) {
             constexpr int ODT = decltype(out_dt_c)::value;
@@ -604,6 +605,21 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
                 pk[g][0] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
                 pk[g][1] = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
             }
+            if (ep.out_scale) {  // block-uniform: fp32 output, every value through e4m3fn on the stored scale and back
+                float* frow = reinterpret_cast<float*>(out) + (int64_t)m * ldo;
+                if (m_ok) {
+#pragma unroll
+                    for (int g = 0; g < 4; g++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const int n = nb + 8 * g + 4 * khalf + e;
+                            const uint16_t h16 = (uint16_t)(pk[g][e >> 1] >> (16 * (e & 1)));
+                            const float f = ep.out_dtype == LLMQ_BF16 ? Lo<LLMQ_BF16>::to_f32(h16) : Lo<LLMQ_F16>::to_f32(h16);
+                            if (n < N) frow[n] = fp8_round_trip(f, out_scale);
+                        }
+                }
+                continue;
+            }
             uint16_t* orow = reinterpret_cast<uint16_t*>(out) + (int64_t)m * ldo;
             if (full && out_vec) {
                 // quads 2g and 2g+1 are exchanged between the half-waves: the lower half ends up with
@@ -658,7 +674,13 @@ __global__ __launch_bounds__(256) void splitk_epilogue_kernel(const void* __rest
         }
         const float sa = ep.a_scale ? ep.a_scale[m] : 1.f, sw = ep.w_scale ? ep.w_scale[n] : 1.f;
         const float bb = ep.bias ? ep.beta * load_as_f32(ep.bias, ep.bias_dtype, n) : 0.f;
-        reinterpret_cast<uint16_t*>(out)[(int64_t)m * ldo + n] = to_out((!ep.bias && alpha == 1.0f) ? epi_value<true>(accf, sa, sw, alpha, 0.f) : epi_value<false>(accf, sa, sw, alpha, bb), ep.out_dtype);
+        const uint16_t h16 = to_out((!ep.bias && alpha == 1.0f) ? epi_value<true>(accf, sa, sw, alpha, 0.f) : epi_value<false>(accf, sa, sw, alpha, bb), ep.out_dtype);
+        if (ep.out_scale) {
+            const float f = ep.out_dtype == LLMQ_BF16 ? Lo<LLMQ_BF16>::to_f32(h16) : Lo<LLMQ_F16>::to_f32(h16);
+            reinterpret_cast<float*>(out)[(int64_t)m * ldo + n] = fp8_round_trip(f, *ep.out_scale);
+        } else {
+            reinterpret_cast<uint16_t*>(out)[(int64_t)m * ldo + n] = h16;
+        }
     }
 }
 

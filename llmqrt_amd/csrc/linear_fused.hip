@@ -109,8 +109,8 @@ __global__ __launch_bounds__(NW * kWave) void linear_fused_kernel(FusedArgs a) {
             cache[c] = i < nchunk ? row[i] : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
-        for (int c = 0; c < kRowChunks; c++) amax = fmaxf(amax, absmax8(cache[c], DT == LLMQ_BF16));
-        for (int i = lane + kRowChunks * kWave; i < nchunk; i += kWave) amax = fmaxf(amax, absmax8(row[i], DT == LLMQ_BF16));
+        for (int c = 0; c < kRowChunks; c++) amax = max_nonneg(amax, absmax8(cache[c], DT == LLMQ_BF16));
+        for (int i = lane + kRowChunks * kWave; i < nchunk; i += kWave) amax = max_nonneg(amax, absmax8(row[i], DT == LLMQ_BF16));
         amax = wave_max(amax);
         const float s = scale_from_amax<DT, MODE>(amax), inv_s = 1.0f / s;
         if (lane == 0) {
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(NW * kWave) void linear_fused_kernel(FusedArgs a) {
     }
 }
 
-int g_force_fused_variant = -1;  // tuning hook: 0 = 2 channel tiles x 4 wavefronts, 1 = 1 x 8
+thread_local int g_force_fused_variant = -1;  // tuning hook (per host thread): 0 = 2 channel tiles x 4 wavefronts, 1 = 1 x 8
 
 template <bool FP8, int DT>
 int launch_fused(const FusedArgs& a, hipStream_t st) {

@@ -40,6 +40,18 @@ __device__ __forceinline__ float epi_value(float acc, float sa, float sw, float 
     return r;
 }
 
+// Round trip of a finished output value through e4m3fn on a stored per-tensor scale, the reference's
+// `static_per_tensor_quantize(output, output_scale).to(dtype) * output_scale`
+// (nn_models/modules/linear/linear_fp8.py:309-311): f is the output already rounded to its 16-bit type; the quotient by
+// the fp32 scale is an fp32 division (a tensor / fp32 tensor promotes), clamped with NaN kept, narrowed to e4m3fn
+// (round to nearest even), widened again (exact) and multiplied by the scale in fp32.
+__device__ __forceinline__ float fp8_round_trip(float f, float s) {
+    const float q = f / s;
+    const float c = (q != q) ? q : __builtin_amdgcn_fmed3f(q, -448.f, 448.f);
+    const int code = __builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false);
+    return __builtin_amdgcn_cvt_f32_fp8(code, 0) * s;
+}
+
 // 16-byte store of finished output with the non-temporal hint: the tile is not read again by this kernel, and
 // without the hint its lines are allocated in L2 beside the operand panels the other tiles of the XCD still need
 // (measured on 8192 x 37888 x 3584: 1177 -> 1042 us, the same as storing into a cache-resident dummy region).
@@ -54,13 +66,22 @@ __device__ __forceinline__ float load_as_f32(const void* p, int dtype, int64_t i
 }
 
 // ---- wavefront / block reductions ---------------------------------------------------------
+// Maximum of two values that are not negative (absolute values, flags), taken on the bit patterns: those order like
+// the values, and a NaN (sign bit clear) is above every number, so it survives every step of a reduction the way
+// torch's max / amax propagate it; fmaxf would drop it.
+__device__ __forceinline__ float max_nonneg(float a, float b) {
+    const uint32_t x = __float_as_uint(a), y = __float_as_uint(b);
+    return __uint_as_float(x > y ? x : y);
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    for (int o = 32; o > 0; o >>= 1) v = max_nonneg(v, __shfl_xor(v, o, kWave));
     return v;
 }
 
-// max over a block of NW wavefronts; every thread gets the result.  `smem` holds NW floats.
+// max over a block of NW wavefronts (non-negative values, NaN propagates); every thread gets the result.
+// `smem` holds NW floats.
 template <int NW>
 __device__ __forceinline__ float block_max(float v, float* smem) {
     v = wave_max(v);
@@ -70,7 +91,7 @@ __device__ __forceinline__ float block_max(float v, float* smem) {
     __syncthreads();
     float r = smem[0];
 #pragma unroll
-    for (int i = 1; i < NW; i++) r = fmaxf(r, smem[i]);
+    for (int i = 1; i < NW; i++) r = max_nonneg(r, smem[i]);
     return r;
 }
 

@@ -26,7 +26,7 @@ template <int DT, int MODE, int SCALE, int NC>
 __global__ __launch_bounds__(kThreads) void quant_rows_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, int64_t K, uint8_t* __restrict__ q,
     void* __restrict__ scale_out, int scale_dtype, const float* __restrict__ aux, int n_aux,
-    int static_f32) {
+    int static_f32, float floor) {
     __shared__ float smem[kNW];
     const int64_t row = blockIdx.x;
     const int tid = threadIdx.x;
@@ -46,18 +46,18 @@ __global__ __launch_bounds__(kThreads) void quant_rows_kernel(
                 cache[c] = (i < nchunk) ? xr[i] : make_uint4(0, 0, 0, 0);
             }
 #pragma unroll
-            for (int c = 0; c < NC; c++) amax = fmaxf(amax, absmax8(cache[c], DT == LLMQ_BF16));
+            for (int c = 0; c < NC; c++) amax = max_nonneg(amax, absmax8(cache[c], DT == LLMQ_BF16));
         } else {
-            for (int i = tid; i < nchunk; i += kThreads) amax = fmaxf(amax, absmax8(xr[i], DT == LLMQ_BF16));
+            for (int i = tid; i < nchunk; i += kThreads) amax = max_nonneg(amax, absmax8(xr[i], DT == LLMQ_BF16));
         }
         amax = block_max<kNW>(amax, smem);
-        s = scale_from_amax<DT, MODE>(amax);
+        s = scale_from_amax<DT, MODE>(amax, floor);
         fin = amax < __builtin_inff() && s > 0.f;  // (the fp8 floor rounds to 0 in fp16: an all-zero row has scale 0 and 0 / 0)
     } else if (SCALE == SCALE_TENSOR) {
         float amax = 0.f;
-        for (int i = tid; i < n_aux; i += kThreads) amax = fmaxf(amax, aux[i]);
+        for (int i = tid; i < n_aux; i += kThreads) amax = max_nonneg(amax, aux[i]);
         amax = block_max<kNW>(amax, smem);
-        s = scale_from_amax<DT, MODE>(amax);
+        s = scale_from_amax<DT, MODE>(amax, floor);
         fin = amax < __builtin_inff() && s > 0.f;  // (the fp8 floor rounds to 0 in fp16: an all-zero row has scale 0 and 0 / 0)
     } else {
         s = aux[0];
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(kThreads) void quant_rows_kernel(
 template <int DT, int MODE, int NCW>
 __global__ __launch_bounds__(kThreads) void quant_rows_wave_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, int64_t K, int64_t M, uint8_t* __restrict__ q,
-    void* __restrict__ scale_out, int scale_dtype) {
+    void* __restrict__ scale_out, int scale_dtype, float floor) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t row = (int64_t)blockIdx.x * kNW + threadIdx.x / kWave;
     if (row >= M) return;  // wavefront-uniform; the kernel has no barrier
@@ -116,9 +116,9 @@ __global__ __launch_bounds__(kThreads) void quant_rows_wave_kernel(
     }
     float amax = 0.f;
 #pragma unroll
-    for (int c = 0; c < NCW; c++) amax = fmaxf(amax, absmax8(cache[c], DT == LLMQ_BF16));
+    for (int c = 0; c < NCW; c++) amax = max_nonneg(amax, absmax8(cache[c], DT == LLMQ_BF16));
     amax = wave_max(amax);
-    const float s = scale_from_amax<DT, MODE>(amax);
+    const float s = scale_from_amax<DT, MODE>(amax, floor);
     if (lane == 0) {
         if (scale_dtype == LLMQ_F32) ((float*)scale_out)[row] = s;
         else ((uint16_t*)scale_out)[row] = Lo<DT>::from_f32(s);
@@ -148,7 +148,7 @@ __global__ __launch_bounds__(kThreads) void absmax_partials_kernel(
     float amax = 0.f;
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kThreads) {
         const int64_t r = i / cpr, c = i - r * cpr;
-        amax = fmaxf(amax, absmax8(reinterpret_cast<const uint4*>(x + r * ldx)[c], DT == LLMQ_BF16));
+        amax = max_nonneg(amax, absmax8(reinterpret_cast<const uint4*>(x + r * ldx)[c], DT == LLMQ_BF16));
     }
     amax = block_max<kNW>(amax, smem);
     if (threadIdx.x == 0) partials[blockIdx.x] = amax;
@@ -237,14 +237,14 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_quant_rows_kernel(
             if (i < nchunk) {
                 cache[c] = norm8<DT>(cache[c], wr[i], inv);
                 if (yr) yr[i] = cache[c];
-                amax = fmaxf(amax, absmax8(cache[c], DT == LLMQ_BF16));
+                amax = max_nonneg(amax, absmax8(cache[c], DT == LLMQ_BF16));
             }
         }
     } else {
         for (int i = tid; i < nchunk; i += kThreads) {
             const uint4 v = norm8<DT>(xr[i], wr[i], inv);
             if (yr) yr[i] = v;
-            amax = fmaxf(amax, absmax8(v, DT == LLMQ_BF16));
+            amax = max_nonneg(amax, absmax8(v, DT == LLMQ_BF16));
         }
     }
     if (QMODE < 0) return;
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_quant_rows_wave_kernel(
         if (i < nchunk) {
             cache[c] = norm8<DT>(cache[c], wr[i], inv);
             if (yr) yr[i] = cache[c];
-            amax = fmaxf(amax, absmax8(cache[c], DT == LLMQ_BF16));
+            amax = max_nonneg(amax, absmax8(cache[c], DT == LLMQ_BF16));
         }
     }
     if (QMODE < 0) return;
@@ -392,7 +392,7 @@ int check_common(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, 
 
 template <int DT, int MODE, int SCALE>
 int launch_rows(const void* x, int64_t M, int64_t K, int64_t ldx, void* q, void* scale, int scale_dtype,
-                const float* aux, int n_aux, int static_f32, hipStream_t st) {
+                const float* aux, int n_aux, int static_f32, float floor, hipStream_t st) {
     const dim3 grid((unsigned)M), block(kThreads);
     const uint16_t* xp = (const uint16_t*)x;
     uint8_t* qp = (uint8_t*)q;
@@ -401,14 +401,14 @@ int launch_rows(const void* x, int64_t M, int64_t K, int64_t ldx, void* q, void*
         const dim3 wgrid((unsigned)((M + kNW - 1) / kNW));
         const int64_t per_lane = ((K >> 3) + kWave - 1) / kWave;
 #define LLMQ_LAUNCH_NCW(NCW) \
-    hipLaunchKernelGGL((quant_rows_wave_kernel<DT, MODE, NCW>), wgrid, block, 0, st, xp, ldx, K, M, qp, scale, scale_dtype)
+    hipLaunchKernelGGL((quant_rows_wave_kernel<DT, MODE, NCW>), wgrid, block, 0, st, xp, ldx, K, M, qp, scale, scale_dtype, floor)
         if (per_lane <= 1) LLMQ_LAUNCH_NCW(1);
         else LLMQ_LAUNCH_NCW(2);
 #undef LLMQ_LAUNCH_NCW
         return launch_status();
     }
 #define LLMQ_LAUNCH_NC(NC) \
-    hipLaunchKernelGGL((quant_rows_kernel<DT, MODE, SCALE, NC>), grid, block, 0, st, xp, ldx, K, qp, scale, scale_dtype, aux, n_aux, static_f32)
+    hipLaunchKernelGGL((quant_rows_kernel<DT, MODE, SCALE, NC>), grid, block, 0, st, xp, ldx, K, qp, scale, scale_dtype, aux, n_aux, static_f32, floor)
     if (SCALE != SCALE_ROW) LLMQ_LAUNCH_NC(0);
     else if (per_thread <= 1) LLMQ_LAUNCH_NC(1);
     else if (per_thread <= 2) LLMQ_LAUNCH_NC(2);
@@ -421,15 +421,15 @@ int launch_rows(const void* x, int64_t M, int64_t K, int64_t ldx, void* q, void*
 
 template <int MODE, int SCALE>
 int dispatch_rows(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, void* q, void* scale,
-                  int scale_dtype, const float* aux, int n_aux, int static_f32, hipStream_t st) {
+                  int scale_dtype, const float* aux, int n_aux, int static_f32, float floor, hipStream_t st) {
     if (x_dtype == LLMQ_BF16)
-        return launch_rows<LLMQ_BF16, MODE, SCALE>(x, M, K, ldx, q, scale, scale_dtype, aux, n_aux, static_f32, st);
-    return launch_rows<LLMQ_F16, MODE, SCALE>(x, M, K, ldx, q, scale, scale_dtype, aux, n_aux, static_f32, st);
+        return launch_rows<LLMQ_BF16, MODE, SCALE>(x, M, K, ldx, q, scale, scale_dtype, aux, n_aux, static_f32, floor, st);
+    return launch_rows<LLMQ_F16, MODE, SCALE>(x, M, K, ldx, q, scale, scale_dtype, aux, n_aux, static_f32, floor, st);
 }
 
 template <int MODE>
 int per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, void* q, void* scale,
-               int scale_dtype, void* ws, size_t ws_bytes, hipStream_t st) {
+               int scale_dtype, void* ws, size_t ws_bytes, float floor, hipStream_t st) {
     if (!ws || ws_bytes < kMaxPartials * sizeof(float)) return LLMQ_ERR_WORKSPACE;
     const int64_t total = M * (K >> 3);
     int nblk = (int)((total + kThreads * 4 - 1) / (kThreads * 4));
@@ -442,7 +442,7 @@ int per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx, vo
         hipLaunchKernelGGL((absmax_partials_kernel<LLMQ_F16>), dim3(nblk), dim3(kThreads), 0, st,
                            (const uint16_t*)x, ldx, M, K, partials);
     if (launch_status() != LLMQ_OK) return LLMQ_ERR_LAUNCH;
-    return dispatch_rows<MODE, SCALE_TENSOR>(x, x_dtype, M, K, ldx, q, scale, scale_dtype, partials, nblk, 0, st);
+    return dispatch_rows<MODE, SCALE_TENSOR>(x, x_dtype, M, K, ldx, q, scale, scale_dtype, partials, nblk, 0, floor, st);
 }
 
 // Per-output-channel int8 weight quantizer (an offline step: one pass when a module is built).  One block per
@@ -465,16 +465,8 @@ __global__ __launch_bounds__(kThreads) void quant_weight_rows_kernel(const void*
     __shared__ float smem[kNW];
     const int64_t row = blockIdx.x;
     float amax = 0.f;
-    bool has_nan = false;
-    for (int64_t k = threadIdx.x; k < K; k += kThreads) {
-        const float v = wq_load<DT>(w, row * ldw + k);
-        has_nan |= (v != v);
-        amax = fmaxf(amax, fabsf(v));
-    }
-    if (has_nan) amax = __builtin_nanf("");  // torch's max propagates NaN
-    float m = block_max<kNW>(has_nan ? __builtin_inff() : amax, smem);
-    const float any_nan = block_max<kNW>(has_nan ? 1.f : 0.f, smem);
-    if (any_nan > 0.f) m = __builtin_nanf("");
+    for (int64_t k = threadIdx.x; k < K; k += kThreads) amax = max_nonneg(amax, fabsf(wq_load<DT>(w, row * ldw + k)));
+    const float m = block_max<kNW>(amax, smem);  // NaN if the row holds one, as torch's max
     const float s = wq_round<DT>(m / 127.f);
     if (threadIdx.x == 0) {
         if (DT == LLMQ_F32) reinterpret_cast<float*>(scale_out)[row] = s;
@@ -496,25 +488,40 @@ extern "C" size_t llmq_quant_workspace_bytes(void) { return kMaxPartials * sizeo
 
 extern "C" int llmq_quant_i8_per_token(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
                                        int8_t* q, void* scale, int scale_dtype, llmq_stream_t stream) {
+    return llmq_quant_i8_per_token_floor(x, x_dtype, M, K, ldx, q, scale, scale_dtype, QP<MODE_I8>::floor_, stream);
+}
+
+extern "C" int llmq_quant_i8_per_token_floor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                             int8_t* q, void* scale, int scale_dtype, float absmax_floor,
+                                             llmq_stream_t stream) {
+    if (!(absmax_floor >= 0.f)) return LLMQ_ERR_SHAPE;
     int rc = check_common(x, x_dtype, M, K, ldx, q);
     if (rc != LLMQ_OK) return rc;
     if (M == 0) return LLMQ_OK;
     if (!scale) return LLMQ_ERR_NULL;
     if (scale_dtype != x_dtype && scale_dtype != LLMQ_F32) return LLMQ_ERR_DTYPE;
     if (K == 0) return LLMQ_ERR_SHAPE;
-    return dispatch_rows<MODE_I8, SCALE_ROW>(x, x_dtype, M, K, ldx, q, scale, scale_dtype, nullptr, 0, 0,
+    return dispatch_rows<MODE_I8, SCALE_ROW>(x, x_dtype, M, K, ldx, q, scale, scale_dtype, nullptr, 0, 0, absmax_floor,
                                              (hipStream_t)stream);
 }
 
 extern "C" int llmq_quant_i8_per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
                                         int8_t* q, void* scale, int scale_dtype, void* workspace,
                                         size_t workspace_bytes, llmq_stream_t stream) {
+    return llmq_quant_i8_per_tensor_floor(x, x_dtype, M, K, ldx, q, scale, scale_dtype, QP<MODE_I8>::floor_, workspace,
+                                          workspace_bytes, stream);
+}
+
+extern "C" int llmq_quant_i8_per_tensor_floor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
+                                              int8_t* q, void* scale, int scale_dtype, float absmax_floor,
+                                              void* workspace, size_t workspace_bytes, llmq_stream_t stream) {
+    if (!(absmax_floor >= 0.f)) return LLMQ_ERR_SHAPE;
     int rc = check_common(x, x_dtype, M, K, ldx, q);
     if (rc != LLMQ_OK) return rc;
     if (!scale) return LLMQ_ERR_NULL;
     if (scale_dtype != x_dtype && scale_dtype != LLMQ_F32) return LLMQ_ERR_DTYPE;
     if (M == 0 || K == 0) return LLMQ_ERR_SHAPE;
-    return per_tensor<MODE_I8>(x, x_dtype, M, K, ldx, q, scale, scale_dtype, workspace, workspace_bytes,
+    return per_tensor<MODE_I8>(x, x_dtype, M, K, ldx, q, scale, scale_dtype, workspace, workspace_bytes, absmax_floor,
                                (hipStream_t)stream);
 }
 
@@ -526,7 +533,7 @@ extern "C" int llmq_quant_fp8_per_token(const void* x, int x_dtype, int64_t M, i
     if (!scale) return LLMQ_ERR_NULL;
     if (K == 0) return LLMQ_ERR_SHAPE;
     return dispatch_rows<MODE_F8, SCALE_ROW>(x, x_dtype, M, K, ldx, q, scale, LLMQ_F32, nullptr, 0, 0,
-                                             (hipStream_t)stream);
+                                             QP<MODE_F8>::floor_, (hipStream_t)stream);
 }
 
 extern "C" int llmq_quant_fp8_per_tensor(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
@@ -537,7 +544,7 @@ extern "C" int llmq_quant_fp8_per_tensor(const void* x, int x_dtype, int64_t M, 
     if (!scale) return LLMQ_ERR_NULL;
     if (M == 0 || K == 0) return LLMQ_ERR_SHAPE;
     return per_tensor<MODE_F8>(x, x_dtype, M, K, ldx, q, scale, LLMQ_F32, workspace, workspace_bytes,
-                               (hipStream_t)stream);
+                               QP<MODE_F8>::floor_, (hipStream_t)stream);
 }
 
 extern "C" int llmq_quant_fp8_static(const void* x, int x_dtype, int64_t M, int64_t K, int64_t ldx,
@@ -548,7 +555,7 @@ extern "C" int llmq_quant_fp8_static(const void* x, int x_dtype, int64_t M, int6
     if (M == 0 || K == 0) return LLMQ_OK;
     if (!scale) return LLMQ_ERR_NULL;
     return dispatch_rows<MODE_F8, SCALE_STATIC>(x, x_dtype, M, K, ldx, q, nullptr, LLMQ_F32, scale, 1,
-                                                scale_is_f32_tensor ? 1 : 0, (hipStream_t)stream);
+                                                scale_is_f32_tensor ? 1 : 0, 0.f, (hipStream_t)stream);
 }
 
 extern "C" int llmq_quant_i8_weight_per_channel(const void* w, int w_dtype, int64_t N, int64_t K, int64_t ldw,

@@ -14,10 +14,12 @@ template <int MODE> struct QP;
 template <> struct QP<MODE_I8> { static constexpr float floor_ = 1e-5f, qmax = 127.f, lo = -128.f, hi = 127.f; };
 template <> struct QP<MODE_F8> { static constexpr float floor_ = 1e-12f, qmax = 448.f, lo = -448.f, hi = 448.f; };
 
+// floor: the lower clamp bound of the absmax (1e-5 / 1e-12 in the Linear modules' quantizers, 1e-8 in the reference's
+// utils/quantization_utils.py:57-71); it lives in the activation dtype, like every other value of the chain.
 template <int DT, int MODE>
-__device__ __forceinline__ float scale_from_amax(float amax) {
-    const float fl = Lo<DT>::round(QP<MODE>::floor_);  // the clamp bound lives in the activation dtype
-    return Lo<DT>::round(fmaxf(amax, fl) / QP<MODE>::qmax);
+__device__ __forceinline__ float scale_from_amax(float amax, float floor = QP<MODE>::floor_) {
+    const float fl = Lo<DT>::round(floor);
+    return Lo<DT>::round(max_nonneg(amax, fl) / QP<MODE>::qmax);  // a NaN absmax stays NaN, as under torch.clamp
 }
 
 typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
@@ -25,7 +27,8 @@ typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float absmax8(uint4 r, int dt_is_bf16) {
     // |x| of 8 packed 16-bit floats.  With the sign bits cleared the bit patterns of bf16 / fp16 values
     // order like the values themselves, so the maximum is taken on packed unsigned 16-bit integers
-    // (two elements per instruction) and only the winner is widened to fp32.
+    // (two elements per instruction) and only the winner is widened to fp32.  A NaN pattern is above every number's, so
+    // a chunk that holds one returns NaN.
     const u16x2 a = __builtin_bit_cast(u16x2, r.x & 0x7fff7fffu), b = __builtin_bit_cast(u16x2, r.y & 0x7fff7fffu);
     const u16x2 c = __builtin_bit_cast(u16x2, r.z & 0x7fff7fffu), d = __builtin_bit_cast(u16x2, r.w & 0x7fff7fffu);
     const u16x2 m = __builtin_elementwise_max(__builtin_elementwise_max(a, b), __builtin_elementwise_max(c, d));
@@ -48,8 +51,9 @@ __device__ __forceinline__ float quotient(float x, float s, float inv_s) {
     return Lo<DT>::round(x * inv_s);
 }
 
-// FIN: the caller knows that no quotient can be NaN (the row's absmax is finite, so every element is finite, and the
-// scale is positive): the per-element NaN handling, which then never fires, is left out.
+// FIN: the caller knows that no quotient can be NaN (the row's absmax, reduced so that a NaN element makes it NaN, is
+// finite, so every element is finite, and the scale is positive): the per-element NaN handling, which then never
+// fires, is left out.
 template <int DT, int MODE, int QUOT, bool FIN = false>
 __device__ __forceinline__ uint2 quant8(uint4 raw, float s, float inv_s) {
     const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};

@@ -11,7 +11,8 @@ import torch
 
 from ..quantize import per_tensor_quantize, per_token_quantize, static_per_tensor_quantize
 from ..sq_fp8_kernels import (cutlass_f8f8bf16_rowwise_sm89, cutlass_f8f8bf16_tensorwise_sm89,
-                              dynamic_linear_max_tokens, f8f8bf16_linear_dynamic_per_token)
+                              dynamic_linear_max_tokens, f8f8_tensorwise_quantized_output,
+                              f8f8bf16_linear_dynamic_per_token)
 from .linear_base import LinearBase
 from .linear_sq import ONE_LAUNCH_MAX_TOKENS, _fusable
 
@@ -37,6 +38,15 @@ class _FP8LinearBase(LinearBase):
         else:
             self.bias = None
         self._q_cache = None
+        self._s_cache = None
+
+    def _wscale_flat(self):
+        """The per-channel weight scales as a contiguous fp32 [N] vector, made once and kept like the fp8 weight."""
+        s = self.weight_scale
+        key = (id(s), s.data_ptr(), s._version, s.device)
+        if self._s_cache is None or self._s_cache[0] != key:
+            self._s_cache = (key, s.detach().to(torch.float32).reshape(-1).contiguous())
+        return self._s_cache[1]
 
     def _qweight_t(self):
         """[K, N] column-major fp8 view of the weight.  The cast is made once and kept until the parameter is
@@ -49,15 +59,16 @@ class _FP8LinearBase(LinearBase):
         return self._q_cache[1].t()
 
     def invalidate_cache(self):
-        """Drop the cached fp8 copy of the weight; the next forward casts again."""
+        """Drop the cached fp8 copy of the weight and the flat copy of its scales; the next forward makes them again."""
         self._q_cache = None
+        self._s_cache = None
 
     def _load_from_state_dict(self, *args, **kwargs):
-        self._q_cache = None   # loaders fill parameters through .data.copy_(), which bumps no version
+        self._q_cache = self._s_cache = None   # loaders fill parameters through .data.copy_(), which bumps no version
         return super()._load_from_state_dict(*args, **kwargs)
 
     def _apply(self, fn, *args, **kwargs):
-        self._q_cache = None   # .to() / .cuda() / .half() replace or rewrite the parameter storage
+        self._q_cache = self._s_cache = None   # .to() / .cuda() / .half() replace or rewrite the parameter storage
         return super()._apply(fn, *args, **kwargs)
 
 
@@ -101,10 +112,10 @@ class FP8DynamicLinear(_FP8LinearBase):
                                                       dtype_to_str.get(self.dtype))
         else:
             x2 = x.reshape(-1, x_shape[-1])
-            if x2.shape[0] <= min(ONE_LAUNCH_MAX_TOKENS, dynamic_linear_max_tokens(x2.shape[-1])) and _fusable(x2):
+            if (self.qdtype == torch.float8_e4m3fn and _fusable(x2)
+                    and x2.shape[0] <= min(ONE_LAUNCH_MAX_TOKENS, dynamic_linear_max_tokens(x2.shape[-1]))):
                 # a few tokens: quantizer and GEMM in one launch (same bits as the two calls below)
-                output = f8f8bf16_linear_dynamic_per_token(x2, qweight, self.bias,
-                                                           self.weight_scale.to(torch.float32).reshape(-1).contiguous())
+                output = f8f8bf16_linear_dynamic_per_token(x2, qweight, self.bias, self._wscale_flat())
                 return output.view(*x_shape[:-1], -1)
             qinput, x_scale = per_token_quantize(x)
             output = cutlass_f8f8bf16_rowwise_sm89(qinput.view(-1, x_shape[-1]), qweight, self.bias,
@@ -159,10 +170,12 @@ class FP8StaticLinear(_FP8LinearBase):
         assert self.per_tensor, "[error!!] static activation quant only support per tensor!"
         qinput = static_per_tensor_quantize(x, self.input_scale)
         alpha = self.weight_scale * self.input_scale
-        output = cutlass_f8f8bf16_tensorwise_sm89(qinput.view(-1, x_shape[-1]), self._qweight_t(), self.bias, alpha,
-                                                  1.0, dtype_to_str.get(self.dtype))
-        output = output.view(*x_shape[:-1], -1)
         if self.quantize_output:
-            qoutput = static_per_tensor_quantize(output, self.output_scale)
-            output = qoutput.to(output.dtype) * self.output_scale
-        return output
+            # output / output_scale -> e4m3fn -> * output_scale (linear_fp8.py:309-311) inside the GEMM epilogue:
+            # one launch, fp32 result as the reference's `qoutput.to(dtype) * output_scale`
+            output = f8f8_tensorwise_quantized_output(qinput.view(-1, x_shape[-1]), self._qweight_t(), self.bias, alpha,
+                                                      1.0, dtype_to_str.get(self.dtype), self.output_scale)
+        else:
+            output = cutlass_f8f8bf16_tensorwise_sm89(qinput.view(-1, x_shape[-1]), self._qweight_t(), self.bias, alpha,
+                                                      1.0, dtype_to_str.get(self.dtype))
+        return output.view(*x_shape[:-1], -1)

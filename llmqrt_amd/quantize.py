@@ -27,16 +27,30 @@ def _as_rows(t: torch.Tensor) -> torch.Tensor:
     return x
 
 
-def _int8_per_token(t: torch.Tensor, scale_dtype):
+def _int8_per_token(t: torch.Tensor, scale_dtype, floor: float = 1e-5):
     x = _as_rows(t)
     M, K = x.shape
     q = torch.empty((M, K), dtype=torch.int8, device=x.device)
     scale = torch.empty((M, 1), dtype=scale_dtype, device=x.device)
     if M:
-        _abi.check(_abi.lib().llmq_quant_i8_per_token(
+        _abi.check(_abi.lib().llmq_quant_i8_per_token_floor(
             x.data_ptr(), _abi.dtype_code(x.dtype), M, K, x.stride(0) if M > 1 else K, q.data_ptr(),
-            scale.data_ptr(), _abi.dtype_code(scale_dtype), _abi.stream_of(x)), "llmq_quant_i8_per_token")
+            scale.data_ptr(), _abi.dtype_code(scale_dtype), floor, _abi.stream_of(x)), "llmq_quant_i8_per_token_floor")
     return q.view(*t.shape), scale.view(*t.shape[:-1], 1)
+
+
+def _int8_per_tensor(t: torch.Tensor, floor: float):
+    x = _as_rows(t)
+    M, K = x.shape
+    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
+    scale = torch.empty((), dtype=t.dtype, device=x.device)
+    ws_bytes = _abi.lib().llmq_quant_workspace_bytes()
+    ws = _abi.workspaces.get(x.device, ws_bytes)
+    _abi.check(_abi.lib().llmq_quant_i8_per_tensor_floor(
+        x.data_ptr(), _abi.dtype_code(x.dtype), M, K, x.stride(0) if M > 1 else K, q.data_ptr(),
+        scale.data_ptr(), _abi.dtype_code(t.dtype), floor, ws.data_ptr(), ws.numel(), _abi.stream_of(x)),
+        "llmq_quant_i8_per_tensor_floor")
+    return q.view(*t.shape), scale
 
 
 @torch.no_grad()
@@ -56,17 +70,21 @@ def quantize_activation_per_token_absmax_f32(t: torch.Tensor):
 def quantize_activation_per_tensor_absmax(t: torch.Tensor, n_bits: int = 8):
     """-> (int8 tensor like t, 0-dim scale in t.dtype)."""
     assert n_bits == 8
-    x = _as_rows(t)
-    M, K = x.shape
-    q = torch.empty((M, K), dtype=torch.int8, device=x.device)
-    scale = torch.empty((), dtype=t.dtype, device=x.device)
-    ws_bytes = _abi.lib().llmq_quant_workspace_bytes()
-    ws = _abi.workspaces.get(x.device, ws_bytes)
-    _abi.check(_abi.lib().llmq_quant_i8_per_tensor(
-        x.data_ptr(), _abi.dtype_code(x.dtype), M, K, x.stride(0) if M > 1 else K, q.data_ptr(),
-        scale.data_ptr(), _abi.dtype_code(t.dtype), ws.data_ptr(), ws.numel(), _abi.stream_of(x)),
-        "llmq_quant_i8_per_tensor")
-    return q.view(*t.shape), scale
+    return _int8_per_tensor(t, 1e-5)
+
+
+@torch.no_grad()
+def dynamic_quantize_activation_per_token_absmax(t: torch.Tensor):
+    """utils/quantization_utils.py:65-71: the per-token quantizer with the absmax clamped at 1e-8 instead of 1e-5.
+    -> (int8 tensor like t, scales [.., 1] in t.dtype).  The reference also overwrites ``t`` with the rounded
+    quotients (in-place ``div_().round_().clamp_()``); here ``t`` is left as it was."""
+    return _int8_per_token(t, t.dtype, 1e-8)
+
+
+@torch.no_grad()
+def dynamic_quantize_activation_per_tensor_absmax(t: torch.Tensor):
+    """utils/quantization_utils.py:57-62: one global absmax clamped at 1e-8.  -> (int8 like t, 0-dim scale in t.dtype)."""
+    return _int8_per_tensor(t, 1e-8)
 
 
 @torch.no_grad()

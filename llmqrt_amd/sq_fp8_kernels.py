@@ -136,6 +136,40 @@ def cutlass_f8f8bf16_tensorwise_sm89(XQ: torch.Tensor, WQ: torch.Tensor, bias: O
 
 
 @torch.no_grad()
+def f8f8_tensorwise_quantized_output(XQ: torch.Tensor, WQ: torch.Tensor, bias: Optional[torch.Tensor], alpha, beta,
+                                     dtype_str: str, output_scale: torch.Tensor) -> torch.Tensor:
+    """cutlass_f8f8bf16_tensorwise_sm89 followed by the output quantization of FP8StaticLinear.forward
+    (nn_models/modules/linear/linear_fp8.py:309-311) in one launch: the ``dtype_str`` result makes a round trip
+    through e4m3fn on ``output_scale`` (a one-element fp32 GPU tensor) inside the GEMM epilogue.  -> fp32 [M, N],
+    the dtype the reference's ``qoutput.to(dtype) * output_scale`` has.  No counterpart among the reference's ops."""
+    what = "f8f8_tensorwise_quantized_output"
+    _check(XQ.dtype in _FP8_FORMATS, f"{what}: XQ must be float8_e4m3fn or float8_e5m2")
+    _check(WQ.dtype == torch.float8_e4m3fn, f"{what}: WQ must be float8_e4m3fn")
+    M, N, K = _check_operands(XQ, WQ, what)
+    _check(dtype_str in _STR_TO_DTYPE,
+           f"{what}: currently only support bf16 or fp16 output dtype, the passed dtype is {dtype_str}")
+    inter = _STR_TO_DTYPE[dtype_str]
+    _check_bias(bias, WQ, N, (torch.bfloat16, torch.float16), what)
+    if bias is not None:
+        _check(bias.dtype == inter, f"{what}: if bias has value, dtype passed in should same as bias dtype")
+    _check(isinstance(output_scale, torch.Tensor) and output_scale.numel() == 1 and output_scale.dtype == torch.float32
+           and output_scale.device == XQ.device, f"{what}: output_scale must be a one-element fp32 tensor on the GPU")
+    a, a_dev = _scalar(alpha, XQ.device)
+    out = torch.empty((M, N), dtype=torch.float32, device=XQ.device)
+    if M == 0 or N == 0:
+        return out
+    L = _abi.lib()
+    ws = _abi.workspaces.get(XQ.device, L.llmq_gemm_fp8_quantized_output_workspace_bytes(M, N, K))
+    st = L.llmq_gemm_fp8_quantized_output(
+        XQ.data_ptr(), _FP8_FORMATS[XQ.dtype], XQ.stride(0), WQ.data_ptr(), WQ.stride(1), None, None, float(a),
+        _abi.ptr(a_dev), _abi.ptr(bias), _abi.dtype_code(bias.dtype) if bias is not None else _abi.BF16, float(beta),
+        output_scale.data_ptr(), out.data_ptr(), _abi.dtype_code(inter), out.stride(0), M, N, K, _abi.ptr(ws),
+        ws.numel() if ws is not None else 0, _abi.stream_of(XQ))
+    _abi.check(st, "llmq_gemm_fp8_quantized_output")
+    return out
+
+
+@torch.no_grad()
 def cutlass_f8f8bf16_rowwise_sm89(XQ: torch.Tensor, WQ: torch.Tensor, bias: Optional[torch.Tensor],
                                   x_scale: torch.Tensor, w_scale: torch.Tensor, use_fast_accum: bool = True,
                                   *, _acc_dump=None) -> torch.Tensor:

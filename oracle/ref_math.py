@@ -61,6 +61,26 @@ def quantize_activation_per_tensor_absmax(t: torch.Tensor):
 
 
 @torch.no_grad()
+def dynamic_quantize_activation_per_token_absmax(t: torch.Tensor):
+    """utils/quantization_utils.py:65-71: as quantize_activation_per_token_absmax with the clamp at 1e-8
+    (which is 0 in fp16).  The reference works in place on t (div_, round_, clamp_); this restatement returns the same
+    (q, scale) without touching t."""
+    max_val = t.abs().max(dim=-1, keepdim=True)[0]
+    max_val = torch.clamp(max_val, min=1e-8) / 127
+    q = (t / max_val).round().clamp(-128, 127).to(torch.int8)
+    return q, max_val
+
+
+@torch.no_grad()
+def dynamic_quantize_activation_per_tensor_absmax(t: torch.Tensor):
+    """utils/quantization_utils.py:57-62."""
+    max_val = t.abs().max()
+    max_val = torch.clamp(max_val, min=1e-8) / 127
+    q = (t / max_val).round().clamp(-128, 127).to(torch.int8)
+    return q, max_val
+
+
+@torch.no_grad()
 def quantize_weight_per_channel_absmax(w: torch.Tensor, native_dtype: bool = False):
     """utils/quantization_utils.py:27-38 (weights [N, K] -> int8 [N, K], scales [N, 1]).
 

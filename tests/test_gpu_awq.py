@@ -46,14 +46,28 @@ def test_dequant_all_nibble_values(cuda):
     assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
 
+_DECODE_WEIGHTS = {}
+
+
+def _decode_weights(K, N):
+    """One seeded weight set per shape, with the oracle's dequantized copy (shared by the token counts)."""
+    from llmqrt_amd import workloads as W
+    if (K, N) not in _DECODE_WEIGHTS:
+        qw, qz, s = W.awq_weights(N, K, 3000 + K % 1000 + N % 1000, group=128)
+        _DECODE_WEIGHTS[(K, N)] = (qw, qz, s, R.awq_dequantize(qw, qz, s, 128).float())
+    return _DECODE_WEIGHTS[(K, N)]
+
+
+# every cell of the decode workload: qkv, o, gate_up, down of Qwen2-7B (and the Qwen2-0.5B up-projection) x 1, 4, 16, 64
+# tokens, on the plan the library picks by itself
 @pytest.mark.parametrize("M", [1, 4, 16, 64])
-@pytest.mark.parametrize("K,N", [(3584, 4608), (896, 4864)])
+@pytest.mark.parametrize("K,N", [(3584, 4608), (3584, 3584), (3584, 37888), (18944, 3584), (896, 4864)])
 def test_gemm_decode_shapes(cuda, M, K, N):
     from llmqrt_amd import workloads as W
     from llmqrt_amd.awq_kernels import awq_gemm_triton
-    qw, qz, s = W.awq_weights(N, K, 3000 + M, group=128)
+    qw, qz, s, wdeq = _decode_weights(K, N)
     x = W.activations(M, K, 3100 + M, dtype=torch.float16, outliers=False)
-    ref = R.awq_gemm(x, qw, qz, s, 128)
+    ref = (x.float() @ wdeq).half()   # dequantize-then-matmul with fp32 accumulation (R.awq_gemm on the shared copy)
     out = awq_gemm_triton(x.to(cuda), qw.to(cuda), s.to(cuda), qz.to(cuda), split_k_iters=8)
     assert out.dtype == torch.float16 and out.shape == (M, N)
     assert rel_err(out, ref) <= REL_TOL
@@ -308,8 +322,8 @@ def test_decode_kernel_token_slabs(cuda, force_awq_plan, plan, M, K, N):
 @pytest.mark.parametrize("M,K,N", [(4, 3584, 4608), (16, 18944, 3584), (48, 3584, 4608)])
 def test_decode_kernel_in_a_hip_graph(cuda, M, K, N):
     """The few-token kernel ends its K split inside the launch with arrival tickets that return to zero; a captured
-    launch replays on the slots it was captured with.  Every replay, with fresh activations and eager calls (which
-    take other slots) in between, must reproduce the eager result bit for bit."""
+    launch replays on the counters of the workspace it was captured with.  Every replay, with fresh activations and
+    eager calls on the same workspace in between (never at the same time), must reproduce the eager result bit for bit."""
     from llmqrt_amd import _abi, workloads as W
     L = _abi.lib()
     qw, qz, s = (t.to(cuda) for t in W.awq_weights(N, K, 77 + M))
@@ -317,7 +331,8 @@ def test_decode_kernel_in_a_hip_graph(cuda, M, K, N):
     out = torch.empty((M, N), dtype=torch.float16, device=cuda)
     nws = L.llmq_awq_gemm_workspace_bytes(M, N, K)
     assert nws > 0, "the shapes are meant to exercise the K split"
-    wsp = torch.empty(nws, dtype=torch.uint8, device=cuda)
+    wsp = torch.zeros(nws, dtype=torch.uint8, device=cuda)   # the counters at its start are cleared once
+    tb = L.llmq_awq_workspace_ticket_bytes()
 
     def run(stream):
         rc = L.llmq_awq_gemm(x.data_ptr(), K, qw.data_ptr(), s.data_ptr(), qz.data_ptr(), None, out.data_ptr(), M, N, K,
@@ -326,7 +341,7 @@ def test_decode_kernel_in_a_hip_graph(cuda, M, K, N):
 
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
-        run(side.cuda_stream)   # first call on the device outside the capture (looks up the ticket ring once)
+        run(side.cuda_stream)
         side.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=side):
@@ -339,7 +354,8 @@ def test_decode_kernel_in_a_hip_graph(cuda, M, K, N):
         torch.cuda.synchronize()
         eager = out.clone()
         out.zero_()
-        wsp.fill_(0xFF)          # the workspace contents must not matter
+        wsp[tb:].fill_(0xFF)     # the contents behind the counters must not matter
+        assert int(wsp[:tb].max()) == 0, "every call leaves the counters at zero"
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager), f"replay {rep}"
@@ -348,8 +364,8 @@ def test_decode_kernel_in_a_hip_graph(cuda, M, K, N):
 
 
 def test_decode_kernel_on_two_streams_at_once(cuda):
-    """Calls on different streams overlap on the GPU; each takes its own run of arrival tickets (the ring wraps
-    several times here), so every result must equal the one computed alone."""
+    """Calls on different streams overlap on the GPU; each stream has its own workspace, hence its own arrival
+    counters, so every result must equal the one computed alone however long the two streams run side by side."""
     from llmqrt_amd import _abi, workloads as W
     L = _abi.lib()
     K, N = 3584, 4608
@@ -359,7 +375,7 @@ def test_decode_kernel_on_two_streams_at_once(cuda):
     xs = [W.activations(M, K, 900 + i, dtype=torch.float16, outliers=False).to(cuda) for i, M in enumerate(Ms)]
     nws = [L.llmq_awq_gemm_workspace_bytes(M, N, K) for M in Ms]
     assert all(n > 0 for n in nws), "both shapes are meant to split K across blocks"
-    wsp = [torch.empty(n, dtype=torch.uint8, device=cuda) for n in nws]
+    wsp = [torch.zeros(n, dtype=torch.uint8, device=cuda) for n in nws]
     alone = []
     for i, M in enumerate(Ms):
         out = torch.empty((M, N), dtype=torch.float16, device=cuda)

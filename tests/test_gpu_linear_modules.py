@@ -127,6 +127,33 @@ def test_fp8_static_module(cuda, quantize_output):
     assert rel_err(y, dense) <= (0.1 if quantize_output else DENSE_TOL)
 
 
+@pytest.mark.parametrize("dtype_str", ["bfloat16", "float16"])
+@pytest.mark.parametrize("M,N,K", [(23, 264, 512), (300, 392, 1040), (512, 768, 384), (64, 3584, 18944)])
+def test_fp8_output_quantization_in_the_epilogue_is_bit_exact(cuda, M, N, K, dtype_str):
+    """f8f8_tensorwise_quantized_output (one launch) against the reference's three steps on the same GEMM result
+    (linear_fp8.py:309-311): the e4m3fn codes and the fp32 outputs must agree bit for bit, on ragged and interior
+    tiles and with a K split (the last shape)."""
+    from llmqrt_amd.sq_fp8_kernels import cutlass_f8f8bf16_tensorwise_sm89, f8f8_tensorwise_quantized_output
+    dt = {"bfloat16": torch.bfloat16, "float16": torch.float16}[dtype_str]
+    g = torch.Generator().manual_seed(M + N)
+    xq = torch.randn(M, K, generator=g).clamp(-3, 3).to(torch.float8_e4m3fn)
+    wq = torch.randn(N, K, generator=g).clamp(-3, 3).to(torch.float8_e4m3fn)
+    bias = torch.randn(N, generator=g).to(dt)
+    alpha = 0.37 / K ** 0.5
+    plain = cutlass_f8f8bf16_tensorwise_sm89(xq.to(cuda), wq.to(cuda).t(), bias.to(cuda), alpha, 1.0, dtype_str).cpu()
+    out_scale = (plain.float().abs().max() / 600.0).reshape(1)   # some outputs beyond +-448 * scale: the clamp matters
+    fused = f8f8_tensorwise_quantized_output(xq.to(cuda), wq.to(cuda).t(), bias.to(cuda), alpha, 1.0, dtype_str,
+                                             out_scale.to(cuda))
+    assert fused.dtype == torch.float32 and fused.shape == (M, N)
+    q_ref = R.fp8_static_per_tensor_quantize(plain, out_scale)
+    assert (q_ref.float().abs() == 448).any(), "the case is meant to reach the clamp"
+    ref = q_ref.to(dt) * out_scale
+    assert ref.dtype == torch.float32
+    assert torch.equal(fused.cpu().view(torch.int32), ref.view(torch.int32))
+    codes = (fused.cpu() / out_scale).to(torch.float8_e4m3fn)
+    assert torch.equal(codes.view(torch.uint8), q_ref.view(torch.uint8))
+
+
 def test_zero_tokens(cuda):
     """The reference returns zeros of the right shape for an empty batch (linear_fp8.py:288-289, linear_awq.py:98)."""
     from llmqrt_amd.linear import FP8DynamicLinear, FP8StaticLinear, WQLinear_GEMM

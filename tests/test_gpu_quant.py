@@ -187,3 +187,91 @@ def test_sq_per_channel_module_quantizes_its_weight_on_the_gpu(cuda):
     mod = SqW8A8BBF16OBF16PerChannel.from_linear(lin, 8, 0, init_only=False, dtype=torch.bfloat16)
     q_ref, s_ref = R.quantize_weight_per_channel_absmax(lin.weight.data.cpu())
     assert torch.equal(mod.qweight.cpu(), q_ref) and torch.equal(mod.weight_scale.cpu(), s_ref.view(-1))
+
+
+# ---- NaN inputs: torch's max / amax propagate a NaN into the scale, so the whole row (per token) or the whole tensor
+# (per tensor) comes out as NaN scale with zero int8 codes / NaN fp8 codes.  (7, 3584): a block per row with the row
+# in registers; (300, 512): a wavefront per row; (3, 24576): a block per row, second pass re-reading the row.
+NAN_SHAPES = [(7, 3584), (300, 512), (3, 24576)]
+
+
+def _with_nans(M, K, seed, dtype):
+    x = _acts(M, K, seed, dtype)
+    x[0, K // 3] = float("nan")   # one NaN in an otherwise finite row
+    x[1] = float("nan")           # an all-NaN row
+    x[2, 0] = float("nan")
+    x[2, K - 1] = float("-inf")   # NaN beside an infinity
+    return x
+
+
+def _same_with_nans(a, b):
+    a, b = a.float(), b.float()
+    return torch.equal(torch.isnan(a), torch.isnan(b)) and torch.equal(torch.nan_to_num(a, nan=0.0), torch.nan_to_num(b, nan=0.0))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K", NAN_SHAPES)
+def test_nan_elements_make_the_row_nan_like_the_reference(cuda, M, K, dtype):
+    from llmqrt_amd.quantize import per_token_quantize, quantize_activation_per_token_absmax
+    x = _with_nans(M, K, 5 * M + K, dtype)
+    q_ref, s_ref = R.quantize_activation_per_token_absmax(x)
+    assert torch.isnan(s_ref[:3]).all() and not torch.isnan(s_ref[3:]).any() and (q_ref[:3] == 0).all()
+    q, s = quantize_activation_per_token_absmax(x.to(cuda))
+    assert _same_with_nans(s.cpu(), s_ref)
+    assert torch.equal(q.cpu(), q_ref)
+    q8_ref, s8_ref = R.fp8_per_token_quantize(x)
+    assert torch.isnan(q8_ref[:3].float()).all()
+    q8, s8 = per_token_quantize(x.to(cuda))
+    assert _same_with_nans(s8.cpu(), s8_ref)
+    assert _same_with_nans(q8.cpu(), q8_ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_nan_element_per_tensor_like_the_reference(cuda, dtype):
+    from llmqrt_amd.quantize import per_tensor_quantize, quantize_activation_per_tensor_absmax
+    x = _acts(40, 1024, 77, dtype)
+    x[17, 300] = float("nan")
+    q_ref, s_ref = R.quantize_activation_per_tensor_absmax(x)
+    q, s = quantize_activation_per_tensor_absmax(x.to(cuda))
+    assert torch.isnan(s_ref).all() and _same_with_nans(s.cpu(), s_ref) and torch.equal(q.cpu(), q_ref)
+    q8_ref, s8_ref = R.fp8_per_tensor_quantize(x)
+    q8, s8 = per_tensor_quantize(x.to(cuda))
+    assert _same_with_nans(s8.cpu(), s8_ref) and _same_with_nans(q8.cpu(), q8_ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K", [(5, 3584), (260, 1024)])
+def test_nan_element_through_rmsnorm_quant(cuda, M, K, dtype):
+    """A NaN in a row makes its mean square, hence every normalised element, NaN: NaN scale, zero codes."""
+    from llmqrt_amd.norm import rmsnorm_quantize_activation_per_token_absmax
+    x = _acts(M, K, 3 * M + K, dtype)
+    x[1, 5] = float("nan")
+    w = (1.0 + 0.1 * torch.randn(K, generator=torch.Generator().manual_seed(1))).to(dtype)
+    q, s = rmsnorm_quantize_activation_per_token_absmax(x.to(cuda), w.to(cuda), 1e-6)
+    assert torch.isnan(s.cpu().float()[1]).all() and (q.cpu()[1] == 0).all()
+    assert not torch.isnan(s.cpu().float()[0]).any() and not torch.isnan(s.cpu().float()[2:]).any()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K", [(7, 3584), (300, 512), (3, 24576)])
+def test_dynamic_quantizers_with_the_1e8_floor(cuda, M, K, dtype):
+    """The twins of utils/quantization_utils.py:57-71 (clamp at 1e-8).  Rows whose absmax lies between the two
+    floors tell them apart: with 1e-5 they quantize to 0 / +-1, with 1e-8 they use the full int8 range.  (In fp16
+    1e-8 rounds to 0, so an all-zero row divides 0 by 0: NaN scale, zero codes, as in the reference.)"""
+    from llmqrt_amd.quantize import (dynamic_quantize_activation_per_tensor_absmax,
+                                     dynamic_quantize_activation_per_token_absmax, quantize_activation_per_token_absmax)
+    x = _acts(M, K, 17 * M + K, dtype)
+    x[1] = (x[1].float() * 1e-7).to(dtype)   # absmax ~4e-7 (fp16: subnormals)
+    x[2] = 0
+    q_ref, s_ref = R.dynamic_quantize_activation_per_token_absmax(x)
+    keep = x.clone()
+    q, s = dynamic_quantize_activation_per_token_absmax(x.to(cuda))
+    assert _same_with_nans(s.cpu(), s_ref) and torch.equal(q.cpu(), q_ref)
+    assert torch.equal(x.view(torch.int16), keep.view(torch.int16))
+    if dtype == torch.bfloat16:   # (fp16 has no values between the two floors' scales: both round to its smallest steps)
+        q5, _ = quantize_activation_per_token_absmax(x.to(cuda))
+        assert not torch.equal(q5.cpu()[1], q_ref[1]), "the tiny row must tell the two floors apart"
+    tiny = (x.float() * 1e-7).to(dtype)
+    qt_ref, st_ref = R.dynamic_quantize_activation_per_tensor_absmax(tiny)
+    qt, st = dynamic_quantize_activation_per_tensor_absmax(tiny.to(cuda))
+    assert _same_with_nans(st.cpu(), st_ref) and torch.equal(qt.cpu(), qt_ref)
