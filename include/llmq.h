@@ -194,8 +194,9 @@ size_t llmq_gemm_fp8_quantized_output_workspace_bytes(int64_t M, int64_t N, int6
  * results as llmq_gemm_w8a8 without acc_dump / workspace: the split-K partial sums go to a static device array
  * of llmq_gemm_static_scratch_bytes() (32 MiB) that every GPU holds from library load to process exit.  The
  * call allocates nothing (no hipMalloc / hipFree), looks the array's device address up once per device (on the
- * first call there: make that call outside a graph capture) and returns LLMQ_ERR_SCRATCH when
- * llmq_gemm_workspace_bytes(M, N, K) exceeds the array.  All calls on one GPU share the array: two calls that
+ * first call there: make that call outside a graph capture).  Arguments are validated as in llmq_gemm_w8a8; then
+ * LLMQ_ERR_SCRATCH is returned, before any launch, when the partial sums of the K split planned for this int8
+ * problem (splits x M x N x 4 bytes; llmq_gemm_workspace_bytes(M, N, K) is an upper bound) exceed the array.  All calls on one GPU share the array: two calls that
  * overlap in time (different streams) race; calls on one stream are ordered and safe.  Nothing in the array has
  * to start at zero: every partial sum is written before it is read. */
 int llmq_gemm_w8a8_static(const int8_t* A, int64_t lda, const int8_t* B, int64_t ldb,

@@ -227,17 +227,16 @@ extern "C" int llmq_gemm_w8a8_static(const int8_t* A, int64_t lda, const int8_t*
                                      const float* w_scale, float alpha, const float* alpha_dev, const void* bias,
                                      int bias_dtype, float beta, void* out, int out_dtype, int64_t ldo, int64_t M,
                                      int64_t N, int64_t K, llmq_stream_t stream) {
-    int sk_t, sk_nw;
-    if (M > 0 && N > 0 && K > 0 && !skinny_plan(M, N, K, sk_t, sk_nw)) {
-        const Plan p = make_plan(M, N, K);
-        if (p.splits > 1 && (size_t)p.splits * M * N * 4 > kStaticScratchBytes) return LLMQ_ERR_SCRATCH;
-    }
     void* ws = nullptr;
-    const int rc = static_scratch(&ws);
+    int rc = static_scratch(&ws);
     if (rc != LLMQ_OK) return rc;
-    return gemm_entry(0, 0, (const uint8_t*)A, lda, (const uint8_t*)B, ldb, a_scale, w_scale, alpha, alpha_dev,
-                      bias, bias_dtype, beta, out, out_dtype, ldo, M, N, K, nullptr, ws, kStaticScratchBytes,
-                      (hipStream_t)stream);
+    // The common entry validates the arguments first and then checks the partial sums of the plan it is about to
+    // launch (the int8 plan of this problem) against the size it is given: a plan that does not fit the array is
+    // refused there, before any launch.
+    rc = gemm_entry(0, 0, (const uint8_t*)A, lda, (const uint8_t*)B, ldb, a_scale, w_scale, alpha, alpha_dev, bias,
+                    bias_dtype, beta, out, out_dtype, ldo, M, N, K, nullptr, ws, kStaticScratchBytes,
+                    (hipStream_t)stream);
+    return rc == LLMQ_ERR_WORKSPACE ? LLMQ_ERR_SCRATCH : rc;
 }
 
 extern "C" int llmq_gemm_force_plan(int cfg, int splits) {
