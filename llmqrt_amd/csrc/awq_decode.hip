@@ -83,7 +83,9 @@ __device__ __forceinline__ void finish_split_tile(const float* ptile, int M, int
         const int m = idx / tile_q, c4 = idx - m * tile_q;
         const v4f v = *reinterpret_cast<const v4f*>(ptile + m * TILE_CH + 4 * c4);
         float* dst = partials + (int64_t)ks * plane + (int64_t)m * N + tile_n0 + 4 * c4;
-        asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
+        // (the wait states: a 16-byte store reads its data registers after issue, and the compiler does not know that this
+        // statement is a store, so it may place a VALU write of those registers right behind it)
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's coherent stores have completed
     __shared__ int s_last;
