@@ -388,9 +388,11 @@ bool awq_decode_supported(int64_t M, int64_t N, int64_t K, int64_t group) {
 // ~40 arrivals (its ticket is one memory word: arrivals serialize at ~50 ns each), and the fp32 partial sums, written
 // through and read back coherently by the one block that finishes a tile, grow with splits x tokens: the more tokens,
 // the fewer blocks along K and the more K slices inside a block (bytes in flight without more arrivals).
-//   wide N (column tiles alone nearly fill the chip; gate_up): one slice and ~2048 wavefronts up to 4 tokens
-//     (17-20 us), blocks of 6 groups at 5-6 tokens (19.0), 2 slices x 5 groups at 7-8 (19.2), beyond that 4 slices
-//     and no split across blocks (21.9 at 16 tokens; the register-streaming kernel needs 24.1);
+//   wide N (column tiles alone nearly fill the chip; gate_up): one slice and blocks of 6 groups up to 6 tokens
+//     (16.2 / 17.9 us at 1 / 4 tokens; blocks of 4 groups, i.e. 7 splits, measured 17.9 / 20.7 on the same box: the
+//     partial sums and arrivals of the extra splits cost more than their wavefronts bring), 2 slices x 5 groups at
+//     7-8 (19.7), beyond that 4 slices and no split across blocks (22.1 at 16 tokens; the register-streaming kernel
+//     needs 24.1);
 //   long K (down): 4 slices of ~3 groups (12.0 us at one token against 13.9 with one slice; 17.3 at 16);
 //   short K, narrow N (qkv, o): 2 slices of one group up to 4 tokens (6.7 us at one token against 7.5; 8.4 at 4
 //     against 10.8), 4 slices of one group beyond (8.9 at 8, 10.7 at 16 tokens);
@@ -415,8 +417,7 @@ AwqDecodePlan make_awq_decode_plan(int64_t M, int64_t N, int64_t K, int force_cs
         else if (K >= 8192) s = std::min(cdiv_d(groups, 11), fit);
         else s = std::min(cdiv_d(groups, 4), fit);
     } else if (strips >= 128) {
-        if (M <= 4) p.ks = 1, s = (int)std::min<int64_t>(s, std::max<int64_t>(groups / M, 1));
-        else if (M <= 6) p.ks = 1, s = std::min(s, cdiv_d(groups, 6));
+        if (M <= 6) p.ks = 1, s = std::min(s, cdiv_d(groups, 6));
         else if (M <= 8) p.ks = 2, s = std::min(s, cdiv_d(groups, 10));
         else p.ks = 4, s = 1;
     } else if (K >= 8192) {
