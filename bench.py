@@ -704,7 +704,8 @@ def micro():
             raise RuntimeError(f"{fn.__name__}{a} failed with {rc}")
         return val.value
 
-    out = {"micro": True, "mfma_TOPS": {}, "lds_bytes_per_ns_per_cu": {}, "empty_kernel_us": {}, "w4_stream_GBs": {}}
+    out = {"micro": True, "mfma_TOPS": {}, "lds_bytes_per_ns_per_cu": {}, "direct_load_bytes_per_ns_per_cu": {},
+           "empty_kernel_us": {}, "w4_stream_GBs": {}}
     for n in (1, 8, 32):
         out["empty_kernel_us"][f"eager_chain_of_{n}"] = round(call(mb.llmq_mb_launch, 0, n), 2)
         out["empty_kernel_us"][f"graph_replay_of_{n}"] = round(call(mb.llmq_mb_launch, 1, n), 2)
@@ -713,6 +714,9 @@ def micro():
             out["mfma_TOPS"][f"{name}_{dn}"] = round(call(mb.llmq_mb_mfma, kind, data), 1)
     for mode, name in enumerate(("ds_read_b128", "ds_write_b128", "global_load_lds_dwordx4")):
         out["lds_bytes_per_ns_per_cu"][name] = round(call(mb.llmq_mb_lds, mode), 1)
+    for total_mb, where in ((128, "infinity_cache"), (512, "hbm")):
+        for sharing in (1, 2, 4, 8, 32):
+            out["direct_load_bytes_per_ns_per_cu"][f"{where}_{sharing}_blocks_per_line"] = round(call(mb.llmq_mb_share, sharing, total_mb), 1)
     # packed AWQ weights of the Qwen2-7B projections, [K, N/8] int32; rows_per_wave = K / (waves x K splits)
     for pname, K, N in (("qkv", 3584, 4608), ("gate_up", 3584, 37888), ("down", 18944, 3584)):
         for mode, mn in enumerate(("regs", "regs_lds_roundtrip", "load_to_lds")):

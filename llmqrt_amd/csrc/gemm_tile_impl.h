@@ -323,8 +323,16 @@ __global__ __launch_bounds__(C::NT) void gemm_tile_kernel(
         for (int i = 0; i < C::B_LOADS; i++) pb[i] = B + (int64_t)n0 * ldb + k_begin + b_off[i] + (ld_c ^ swz) * 16;
         const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem_raw);
         const uint32_t wave_off = (uint32_t)__builtin_amdgcn_readfirstlane(wave) * 1024u;
+        // int32 accumulators (any summation order gives the same bits): every XCD starts its walk over K at another
+        // eighth and wraps around (blockIdx.x % 8 is the XCD), so the eight L2s ask the fabric for different lines of the
+        // shared panels at any moment instead of all for the same ones.  The blocks of one XCD stay in step, which is what
+        // lets them share a panel through their L2.  fp32 accumulators keep the natural order: their bits would
+        // otherwise depend on where in the grid a tile sits.
+        const int krot = C::FACC ? 0 : (int)((blockIdx.x % kNumXcd) * (unsigned)ktiles / kNumXcd);
         auto issue_tile = [&](int kt, int stage) {
-            const int koff = min(kt, ktiles - 1) * C::BK;  // past the end: the last tile again, into a stage nobody reads
+            int kr = min(kt, ktiles - 1) + krot;  // past the end: the last tile again, into a stage nobody reads
+            kr -= kr >= ktiles ? ktiles : 0;
+            const int koff = kr * C::BK;
             const uint32_t sbase = lds_base + (uint32_t)stage * (C::STAGE_CHUNKS * 16u) + wave_off;
 #pragma unroll
             for (int i = 0; i < C::A_LOADS; i++) {

@@ -8,6 +8,9 @@
 //                   access pattern (128-byte row segments, eight 16-byte loads per lane): short-lived wavefronts
 //                   that request their whole share at once against wavefronts that loop, with the data consumed
 //                   from registers, passed through LDS (as a layout change needs), or loaded straight into LDS.
+//   llmq_mb_share   direct-load (global_load_lds_dwordx4) bandwidth per CU with all 256 CUs streaming, as a function of
+//                   how many blocks of an XCD read the same lines (1 / sharing = the fraction of the requested bytes
+//                   that the XCD's L2 has to fetch from the fabric): the supply side of the GEMM main loops.
 //   llmq_mb_launch  time per kernel of a chain of empty kernels on one stream, launched one by one or replayed
 //                   from a HIP graph: the floor under every short launch of the decode path.
 // Each function allocates what it needs, times its kernel with HIP events and returns 0 on success.
@@ -103,6 +106,31 @@ __global__ __launch_bounds__(512) void lds_kernel(const uint4* __restrict__ src,
     }
     __syncthreads();
     out[blockIdx.x * 512 + tid] = acc + reinterpret_cast<uint32_t*>(smem)[tid] + v.x;
+}
+
+// ---- operand supply: f blocks of an XCD stream one region together (64 KB per block and iteration, 16 KB per
+// wavefront in flight), every region longer than the L2 so that no line is found there a second time -----------------
+__global__ __launch_bounds__(512) void share_kernel(const uint8_t* __restrict__ src, size_t region, int f, int iters, uint32_t* out) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid & 63;
+    const int xcd = blockIdx.x % 8, local = blockIdx.x / 8, group = local / f;  // consecutive block ids go round the XCDs
+    const uint8_t* base = src + (size_t)(xcd * (32 / f) + group) * region;
+    const uint32_t lbase = (uint32_t)(uintptr_t)MB_LPTR(smem) + __builtin_amdgcn_readfirstlane(wave) * 1024u;
+    size_t off = 0;
+    for (int i = 0; i < iters; i++) {
+        const uint8_t* p = base + off + wave * 1024 + lane * 16;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t m0v = lbase + j * 8192u;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0v), "v"(p + j * 8192) : "memory", "m0");
+        }
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        off += 65536;
+        if (off >= region) off = 0;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (iters < 0) out[blockIdx.x] = smem[tid];
 }
 
 // ---- HBM streaming of the packed weight matrix: 128-byte segments, 8 rows per instruction, 8 loads per pass -----
@@ -246,6 +274,27 @@ extern "C" int llmq_mb_lds(int mode, double* bytes_per_ns_per_cu) {
     (void)hipFree(out);
     if (rc) return rc;
     *bytes_per_ns_per_cu = (double)iters * 8192 * 8 / (ms * 1e6);
+    return 0;
+}
+
+// sharing: 1, 2, 4, 8 or 32 blocks of an XCD read the same region.  total_mb: bytes of all regions together (128: they
+// stay in the Infinity Cache; 512: they come from HBM).  -> bytes per nanosecond and CU with 256 blocks running
+extern "C" int llmq_mb_share(int sharing, int total_mb, double* bytes_per_ns_per_cu) {
+    if ((sharing != 1 && sharing != 2 && sharing != 4 && sharing != 8 && sharing != 32) || total_mb < 64 || total_mb > 1024) return 2;
+    const size_t total = (size_t)total_mb << 20, region = total / (256 / sharing);
+    if (region % 65536 != 0) return 2;
+    uint8_t* src;
+    uint32_t* out;
+    MB_CK(hipMalloc(&src, total));
+    MB_CK(hipMemset(src, 1, total));
+    MB_CK(hipMalloc(&out, 256 * 4));
+    const int iters = 8192;
+    float ms;
+    const int rc = time_ms([&] { hipLaunchKernelGGL(share_kernel, dim3(256), dim3(512), 65536, 0, src, region, sharing, iters, out); }, 1, &ms);
+    (void)hipFree(src);
+    (void)hipFree(out);
+    if (rc) return rc;
+    *bytes_per_ns_per_cu = (double)iters * 65536 / (ms * 1e6);
     return 0;
 }
 
