@@ -98,30 +98,62 @@ __device__ __forceinline__ void finish_split_tile(const float* ptile, int M, int
     }
     __syncthreads();
     if (!s_last) return;
-    for (int idx = tid; idx < M * tile_q; idx += NT) {
-        const int m = idx / tile_q, nn = tile_n0 + 4 * (idx - m * tile_q);
-        const float* src = partials + (int64_t)m * N + nn;
-        const int64_t sstride = plane;
-        v4f acc = {0.f, 0.f, 0.f, 0.f};
-        for (int sp = 0; sp < splits; sp += 8) {  // eight coherent loads in flight, added in split order
-            v4f t0, t1, t2, t3, t4, t5, t6, t7;
-            auto ld = [&](int i, v4f& t) __attribute__((always_inline)) {
-                const float* p = src + (int64_t)min(sp + i, splits - 1) * sstride;
-                asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(t) : "v"(p) : "memory");
-            };
-            ld(0, t0), ld(1, t1), ld(2, t2), ld(3, t3), ld(4, t4), ld(5, t5), ld(6, t6), ld(7, t7);
-            asm volatile("s_waitcnt vmcnt(0)" : "+v"(t0), "+v"(t1), "+v"(t2), "+v"(t3), "+v"(t4), "+v"(t5), "+v"(t6), "+v"(t7)::"memory");
-            const int left = splits - sp;
-            acc += t0;
-            if (left > 1) acc += t1;
-            if (left > 2) acc += t2;
-            if (left > 3) acc += t3;
-            if (left > 4) acc += t4;
-            if (left > 5) acc += t5;
-            if (left > 6) acc += t6;
-            if (left > 7) acc += t7;
+    // Eight splits at a time, added in split order.  Every coherent load goes to memory, so the read-back costs one round
+    // trip per pass: where a pass has more pieces than threads (16 tokens on 512 threads), a thread takes two pieces,
+    // sixteen 16-byte loads in flight.
+    const int items = M * tile_q;
+    auto ld = [&](const float* src, int sp, v4f& t) __attribute__((always_inline)) {
+        const float* q = src + (int64_t)min(sp, splits - 1) * plane;
+        asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(t) : "v"(q) : "memory");
+    };
+    auto add8 = [&](v4f& acc, int left, v4f t0, v4f t1, v4f t2, v4f t3, v4f t4, v4f t5, v4f t6, v4f t7) __attribute__((always_inline)) {
+        acc += t0;
+        if (left > 1) acc += t1;
+        if (left > 2) acc += t2;
+        if (left > 3) acc += t3;
+        if (left > 4) acc += t4;
+        if (left > 5) acc += t5;
+        if (left > 6) acc += t6;
+        if (left > 7) acc += t7;
+    };
+    for (int base = 0; base < items; base += 2 * NT) {
+        const int idx = base + tid, idx1 = idx + NT;
+        if (base + NT < items) {  // block-uniform: the second half of the pass is not empty
+            const bool two = idx1 < items;  // a lane without a second piece loads its first one twice
+            const int ia = idx, ib = two ? idx1 : idx;
+            const int ma = ia / tile_q, na = tile_n0 + 4 * (ia - ma * tile_q);
+            const int mb = ib / tile_q, nb = tile_n0 + 4 * (ib - mb * tile_q);
+            const float* srca = partials + (int64_t)ma * N + na;
+            const float* srcb = partials + (int64_t)mb * N + nb;
+            v4f acca = {0.f, 0.f, 0.f, 0.f}, accb = {0.f, 0.f, 0.f, 0.f};
+            for (int sp = 0; sp < splits; sp += 8) {
+                v4f a0, a1, a2, a3, a4, a5, a6, a7, b0, b1, b2, b3, b4, b5, b6, b7;
+                ld(srca, sp, a0), ld(srca, sp + 1, a1), ld(srca, sp + 2, a2), ld(srca, sp + 3, a3);
+                ld(srca, sp + 4, a4), ld(srca, sp + 5, a5), ld(srca, sp + 6, a6), ld(srca, sp + 7, a7);
+                ld(srcb, sp, b0), ld(srcb, sp + 1, b1), ld(srcb, sp + 2, b2), ld(srcb, sp + 3, b3);
+                ld(srcb, sp + 4, b4), ld(srcb, sp + 5, b5), ld(srcb, sp + 6, b6), ld(srcb, sp + 7, b7);
+                asm volatile("s_waitcnt vmcnt(0)"
+                             : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7), "+v"(b0),
+                               "+v"(b1), "+v"(b2), "+v"(b3), "+v"(b4), "+v"(b5), "+v"(b6), "+v"(b7)::"memory");
+                add8(acca, splits - sp, a0, a1, a2, a3, a4, a5, a6, a7);
+                add8(accb, splits - sp, b0, b1, b2, b3, b4, b5, b6, b7);
+            }
+            store4(acca, ma, na);
+            if (two) store4(accb, mb, nb);
+        } else if (idx < items) {
+            const int ia = idx;
+            const int ma = ia / tile_q, na = tile_n0 + 4 * (ia - ma * tile_q);
+            const float* srca = partials + (int64_t)ma * N + na;
+            v4f acca = {0.f, 0.f, 0.f, 0.f};
+            for (int sp = 0; sp < splits; sp += 8) {
+                v4f a0, a1, a2, a3, a4, a5, a6, a7;
+                ld(srca, sp, a0), ld(srca, sp + 1, a1), ld(srca, sp + 2, a2), ld(srca, sp + 3, a3);
+                ld(srca, sp + 4, a4), ld(srca, sp + 5, a5), ld(srca, sp + 6, a6), ld(srca, sp + 7, a7);
+                asm volatile("s_waitcnt vmcnt(0)" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7)::"memory");
+                add8(acca, splits - sp, a0, a1, a2, a3, a4, a5, a6, a7);
+            }
+            store4(acca, ma, na);
         }
-        store4(acc, m, nn);
     }
 }
 
