@@ -12,17 +12,31 @@ constexpr int kWave = 64;  // CDNA wavefront width
 
 // ---- 16-bit float storage types, handled as raw bits + fp32 math -------------------------
 template <int DT> struct Lo;
+typedef float lo_f2 __attribute__((ext_vector_type(2)));
 template <> struct Lo<LLMQ_BF16> {
     static __device__ __forceinline__ float to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
     static __device__ __forceinline__ uint16_t from_f32(float f) {  // round to nearest even
         return __builtin_bit_cast(uint16_t, (__bf16)f);
     }
     static __device__ __forceinline__ float round(float f) { return to_f32(from_f32(f)); }
+    // two values narrowed by one packed conversion: a in the low half, b in the high half
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+        typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(lo_f2{a, b}, bf2));
+    }
+    static __device__ __forceinline__ float lo_f32(uint32_t p) { return __uint_as_float(p << 16); }
+    static __device__ __forceinline__ float hi_f32(uint32_t p) { return __uint_as_float(p & 0xffff0000u); }
 };
 template <> struct Lo<LLMQ_F16> {
     static __device__ __forceinline__ float to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
     static __device__ __forceinline__ uint16_t from_f32(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
     static __device__ __forceinline__ float round(float f) { return to_f32(from_f32(f)); }
+    static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(lo_f2{a, b}, h2));
+    }
+    static __device__ __forceinline__ float lo_f32(uint32_t p) { return to_f32((uint16_t)(p & 0xffffu)); }
+    static __device__ __forceinline__ float hi_f32(uint32_t p) { return to_f32((uint16_t)(p >> 16)); }
 };
 
 // GEMM epilogue value in fp32, each node rounded once: (acc * sa) * sw, then one fused multiply-add with alpha and
@@ -74,9 +88,37 @@ __device__ __forceinline__ float max_nonneg(float a, float b) {
     return __uint_as_float(x > y ? x : y);
 }
 
+// The value of lane (lane ^ O), O a power of two, without an address computation: DPP lane selects inside quads and
+// 16-lane rows, ds_swizzle inside 32 lanes, v_permlane32_swap across the two halves of the wavefront.
+template <int O>
+__device__ __forceinline__ float lane_xor(float v) {
+    const int i = __float_as_int(v);
+    if constexpr (O == 1) return __int_as_float(__builtin_amdgcn_mov_dpp(i, 0xB1, 0xf, 0xf, true));        // quad_perm [1,0,3,2]
+    else if constexpr (O == 2) return __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
+    else if constexpr (O == 4) return __int_as_float(__builtin_amdgcn_ds_swizzle(i, 0x101F));              // xor_mask 4
+    else if constexpr (O == 8) return __int_as_float(__builtin_amdgcn_mov_dpp(i, 0x128, 0xf, 0xf, true));  // row_ror:8
+    else {
+        static_assert(O == 16, "lane distance");
+        return __int_as_float(__builtin_amdgcn_ds_swizzle(i, 0x401F));  // xor_mask 16
+    }
+}
+// Distance 32: v_permlane32_swap of v with itself returns {v with its upper half replaced by its lower half, v with its
+// lower half replaced by its upper half}; in every lane one of the two is the lane's own value and the other its partner's.
+__device__ __forceinline__ void lane_xor32_pair(float v, float& a, float& b) {
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_int(v), __float_as_int(v), false, false);
+    a = __int_as_float(sw[0]);
+    b = __int_as_float(sw[1]);
+}
+
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = max_nonneg(v, __shfl_xor(v, o, kWave));
+    float a, b;
+    lane_xor32_pair(v, a, b);
+    v = max_nonneg(a, b);
+    v = max_nonneg(v, lane_xor<16>(v));
+    v = max_nonneg(v, lane_xor<8>(v));
+    v = max_nonneg(v, lane_xor<4>(v));
+    v = max_nonneg(v, lane_xor<2>(v));
+    v = max_nonneg(v, lane_xor<1>(v));
     return v;
 }
 
@@ -95,9 +137,16 @@ __device__ __forceinline__ float block_max(float v, float* smem) {
     return r;
 }
 
+// butterfly: lane distances 32, 16, 8, 4, 2, 1 in this order; every lane ends with the same bits
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    float a, b;
+    lane_xor32_pair(v, a, b);
+    v = a + b;  // own value + partner's, in either order
+    v += lane_xor<16>(v);
+    v += lane_xor<8>(v);
+    v += lane_xor<4>(v);
+    v += lane_xor<2>(v);
+    v += lane_xor<1>(v);
     return v;
 }
 

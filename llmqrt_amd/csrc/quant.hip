@@ -19,15 +19,15 @@ constexpr int kMaxPartials = 1024;  // per-tensor absmax partials (one per stage
 
 enum { SCALE_ROW = 0, SCALE_TENSOR = 1, SCALE_STATIC = 2 };
 
-// One block per row.  NC > 0: the row's 16-byte chunks (8 elements) are kept in NC
+// One block of NT threads per row.  NC > 0: the row's 16-byte chunks (8 elements) are kept in NC
 // registers per thread between the two passes; NC == 0: rows of any length, second pass
 // re-reads x (served by L2).
-template <int DT, int MODE, int SCALE, int NC>
-__global__ __launch_bounds__(kThreads) void quant_rows_kernel(
+template <int DT, int MODE, int SCALE, int NC, int NT = kThreads>
+__global__ __launch_bounds__(NT) void quant_rows_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, int64_t K, uint8_t* __restrict__ q,
     void* __restrict__ scale_out, int scale_dtype, const float* __restrict__ aux, int n_aux,
     int static_f32, float floor) {
-    __shared__ float smem[kNW];
+    __shared__ float smem[NT / kWave];
     const int64_t row = blockIdx.x;
     const int tid = threadIdx.x;
     const int nchunk = (int)(K >> 3);
@@ -42,21 +42,21 @@ __global__ __launch_bounds__(kThreads) void quant_rows_kernel(
         if (NC > 0) {
 #pragma unroll
             for (int c = 0; c < NC; c++) {
-                const int i = tid + c * kThreads;
+                const int i = tid + c * NT;
                 cache[c] = (i < nchunk) ? xr[i] : make_uint4(0, 0, 0, 0);
             }
 #pragma unroll
             for (int c = 0; c < NC; c++) amax = max_nonneg(amax, absmax8(cache[c], DT == LLMQ_BF16));
         } else {
-            for (int i = tid; i < nchunk; i += kThreads) amax = max_nonneg(amax, absmax8(xr[i], DT == LLMQ_BF16));
+            for (int i = tid; i < nchunk; i += NT) amax = max_nonneg(amax, absmax8(xr[i], DT == LLMQ_BF16));
         }
-        amax = block_max<kNW>(amax, smem);
+        amax = block_max<NT / kWave>(amax, smem);
         s = scale_from_amax<DT, MODE>(amax, floor);
         fin = amax < __builtin_inff() && s > 0.f;  // (the fp8 floor rounds to 0 in fp16: an all-zero row has scale 0 and 0 / 0)
     } else if (SCALE == SCALE_TENSOR) {
         float amax = 0.f;
-        for (int i = tid; i < n_aux; i += kThreads) amax = max_nonneg(amax, aux[i]);
-        amax = block_max<kNW>(amax, smem);
+        for (int i = tid; i < n_aux; i += NT) amax = max_nonneg(amax, aux[i]);
+        amax = block_max<NT / kWave>(amax, smem);
         s = scale_from_amax<DT, MODE>(amax, floor);
         fin = amax < __builtin_inff() && s > 0.f;  // (the fp8 floor rounds to 0 in fp16: an all-zero row has scale 0 and 0 / 0)
     } else {
@@ -73,26 +73,26 @@ __global__ __launch_bounds__(kThreads) void quant_rows_kernel(
         if (fin) {
 #pragma unroll
             for (int c = 0; c < NC; c++) {
-                const int i = tid + c * kThreads;
+                const int i = tid + c * NT;
                 if (i < nchunk) qr[i] = quant8<DT, MODE, Q_DT, true>(cache[c], s, inv_s);
             }
         } else {
 #pragma unroll
             for (int c = 0; c < NC; c++) {
-                const int i = tid + c * kThreads;
+                const int i = tid + c * NT;
                 if (i < nchunk) qr[i] = quant8<DT, MODE, Q_DT>(cache[c], s, inv_s);
             }
         }
     } else if (F32Q) {
         if (static_f32) {
-            for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, MODE, Q_DIV_F32>(xr[i], s, inv_s);
+            for (int i = tid; i < nchunk; i += NT) qr[i] = quant8<DT, MODE, Q_DIV_F32>(xr[i], s, inv_s);
         } else {
-            for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, MODE, Q_DIV_DT>(xr[i], s, inv_s);
+            for (int i = tid; i < nchunk; i += NT) qr[i] = quant8<DT, MODE, Q_DIV_DT>(xr[i], s, inv_s);
         }
     } else if (fin) {
-        for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, MODE, Q_DT, true>(xr[i], s, inv_s);
+        for (int i = tid; i < nchunk; i += NT) qr[i] = quant8<DT, MODE, Q_DT, true>(xr[i], s, inv_s);
     } else {
-        for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, MODE, Q_DT>(xr[i], s, inv_s);
+        for (int i = tid; i < nchunk; i += NT) qr[i] = quant8<DT, MODE, Q_DT>(xr[i], s, inv_s);
     }
 }
 
@@ -184,25 +184,25 @@ __device__ __forceinline__ uint4 norm8(uint4 r, uint4 wv, float inv) {
     for (int i = 0; i < 4; i++) {
         // The reference rounds the product to fp32 and then to the activation dtype.  Keep the fp32 product
         // opaque so that the compiler cannot fuse multiply and narrowing into one mixed-precision
-        // instruction, which rounds once and lands on the other side of a tie now and then.
-        float p0 = Lo<DT>::to_f32((uint16_t)(x[i] & 0xffffu)) * inv;
-        float p1 = Lo<DT>::to_f32((uint16_t)(x[i] >> 16)) * inv;
+        // instruction, which rounds once and lands on the other side of a tie now and then.  The two narrowings of a
+        // pair share one packed conversion.
+        float p0 = Lo<DT>::lo_f32(x[i]) * inv;
+        float p1 = Lo<DT>::hi_f32(x[i]) * inv;
         asm volatile("" : "+v"(p0), "+v"(p1));
-        const float n0 = Lo<DT>::round(p0), n1 = Lo<DT>::round(p1);
-        const uint16_t y0 = Lo<DT>::from_f32(Lo<DT>::to_f32((uint16_t)(w[i] & 0xffffu)) * n0);
-        const uint16_t y1 = Lo<DT>::from_f32(Lo<DT>::to_f32((uint16_t)(w[i] >> 16)) * n1);
-        o[i] = (uint32_t)y0 | ((uint32_t)y1 << 16);
+        const uint32_t n = Lo<DT>::pack2(p0, p1);
+        // (the product of two 16-bit floats is exact in fp32: narrowing it rounds once however it is compiled)
+        o[i] = Lo<DT>::pack2(Lo<DT>::lo_f32(w[i]) * Lo<DT>::lo_f32(n), Lo<DT>::hi_f32(w[i]) * Lo<DT>::hi_f32(n));
     }
     return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
 // QMODE: -1 = no quantizer (plain RMSNorm), MODE_I8, MODE_F8.
-template <int DT, int QMODE, int NC>
-__global__ __launch_bounds__(kThreads) void rmsnorm_quant_rows_kernel(
+template <int DT, int QMODE, int NC, int NT = kThreads>
+__global__ __launch_bounds__(NT) void rmsnorm_quant_rows_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, int64_t K, const uint16_t* __restrict__ weight, float eps,
     uint16_t* __restrict__ y, uint8_t* __restrict__ q, void* __restrict__ scale_out, int scale_dtype,
     float* __restrict__ inv_out) {
-    __shared__ float smem[kNW];
+    __shared__ float smem[NT / kWave];
     constexpr int QM = QMODE < 0 ? MODE_I8 : QMODE;
     const int64_t row = blockIdx.x;
     const int tid = threadIdx.x;
@@ -217,15 +217,15 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_quant_rows_kernel(
     if (NC > 0) {
 #pragma unroll
         for (int c = 0; c < NC; c++) {
-            const int i = tid + c * kThreads;
+            const int i = tid + c * NT;
             cache[c] = (i < nchunk) ? xr[i] : make_uint4(0, 0, 0, 0);
         }
 #pragma unroll
         for (int c = 0; c < NC; c++) ss = sumsq8<DT>(cache[c], ss);
     } else {
-        for (int i = tid; i < nchunk; i += kThreads) ss = sumsq8<DT>(xr[i], ss);
+        for (int i = tid; i < nchunk; i += NT) ss = sumsq8<DT>(xr[i], ss);
     }
-    ss = block_sum<kNW>(ss, smem);
+    ss = block_sum<NT / kWave>(ss, smem);
     const float inv = 1.0f / sqrtf(ss / (float)K + eps);
     if (inv_out && tid == 0) inv_out[row] = inv;
 
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_quant_rows_kernel(
     if (NC > 0) {
 #pragma unroll
         for (int c = 0; c < NC; c++) {
-            const int i = tid + c * kThreads;
+            const int i = tid + c * NT;
             if (i < nchunk) {
                 cache[c] = norm8<DT>(cache[c], wr[i], inv);
                 if (yr) yr[i] = cache[c];
@@ -241,14 +241,14 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_quant_rows_kernel(
             }
         }
     } else {
-        for (int i = tid; i < nchunk; i += kThreads) {
+        for (int i = tid; i < nchunk; i += NT) {
             const uint4 v = norm8<DT>(xr[i], wr[i], inv);
             if (yr) yr[i] = v;
             amax = max_nonneg(amax, absmax8(v, DT == LLMQ_BF16));
         }
     }
     if (QMODE < 0) return;
-    amax = block_max<kNW>(amax, smem);
+    amax = block_max<NT / kWave>(amax, smem);
     const float s = scale_from_amax<DT, QM>(amax);
     if (tid == 0) {
         if (scale_dtype == LLMQ_F32) ((float*)scale_out)[row] = s;
@@ -258,17 +258,17 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_quant_rows_kernel(
     if (NC > 0 && amax < __builtin_inff() && s > 0.f) {  // block-uniform: no quotient can be NaN
 #pragma unroll
         for (int c = 0; c < NC; c++) {
-            const int i = tid + c * kThreads;
+            const int i = tid + c * NT;
             if (i < nchunk) qr[i] = quant8<DT, QM, Q_DT, true>(cache[c], s, inv_s);
         }
     } else if (NC > 0) {
 #pragma unroll
         for (int c = 0; c < NC; c++) {
-            const int i = tid + c * kThreads;
+            const int i = tid + c * NT;
             if (i < nchunk) qr[i] = quant8<DT, QM, Q_DT>(cache[c], s, inv_s);
         }
     } else {
-        for (int i = tid; i < nchunk; i += kThreads) qr[i] = quant8<DT, QM, Q_DT>(norm8<DT>(xr[i], wr[i], inv), s, inv_s);
+        for (int i = tid; i < nchunk; i += NT) qr[i] = quant8<DT, QM, Q_DT>(norm8<DT>(xr[i], wr[i], inv), s, inv_s);
     }
 }
 
@@ -337,6 +337,10 @@ __global__ __launch_bounds__(kThreads) void rmsnorm_quant_rows_wave_kernel(
 // (quantizer) / 9.7 us (RMSNorm + quantizer) against 9.3 / 13.7 us for a block per row; at K = 3584 a block per row is
 // ahead by 5 % (17.2 against 18.0 us) and by 1.3 us at a few rows, so longer rows keep it.
 inline bool wave_rows(int64_t M, int64_t K) { return (K >> 3) <= 2 * kWave && M >= 256; }
+// Rows of 257-512 chunks (K = 3584: 448) with enough rows to fill the chip run on half-size blocks with four chunks
+// per thread: the per-row arithmetic that every wavefront repeats (two reductions, the scale, its reciprocal) is spread
+// over twice the elements.  Fused RMSNorm + int8 quantizer at 8192 x 3584 from HBM: 21.6 us against 23.6.
+inline bool half_blocks(int64_t M, int64_t K) { return (K >> 3) > kThreads && (K >> 3) <= 2 * kThreads && M >= 256; }
 
 template <int DT, int QMODE>
 int launch_norm(const void* x, int64_t M, int64_t K, int64_t ldx, const void* weight, float eps, void* y, void* q,
@@ -354,15 +358,18 @@ int launch_norm(const void* x, int64_t M, int64_t K, int64_t ldx, const void* we
 #undef LLMQ_LAUNCH_NCW
         return launch_status();
     }
-#define LLMQ_LAUNCH_NC(NC)                                                                                      \
-    hipLaunchKernelGGL((rmsnorm_quant_rows_kernel<DT, QMODE, NC>), grid, block, 0, st, (const uint16_t*)x, ldx, K, \
+#define LLMQ_LAUNCH_NCT(NC, NT)                                                                                          \
+    hipLaunchKernelGGL((rmsnorm_quant_rows_kernel<DT, QMODE, NC, NT>), grid, dim3(NT), 0, st, (const uint16_t*)x, ldx, K, \
                        (const uint16_t*)weight, eps, (uint16_t*)y, (uint8_t*)q, scale, scale_dtype, inv_out)
-    if (per_thread <= 1) LLMQ_LAUNCH_NC(1);
+#define LLMQ_LAUNCH_NC(NC) LLMQ_LAUNCH_NCT(NC, kThreads)
+    if (half_blocks(M, K)) LLMQ_LAUNCH_NCT(4, kThreads / 2);
+    else if (per_thread <= 1) LLMQ_LAUNCH_NC(1);
     else if (per_thread <= 2) LLMQ_LAUNCH_NC(2);
     else if (per_thread <= 4) LLMQ_LAUNCH_NC(4);
     else if (per_thread <= 10) LLMQ_LAUNCH_NC(10);
     else LLMQ_LAUNCH_NC(0);
 #undef LLMQ_LAUNCH_NC
+#undef LLMQ_LAUNCH_NCT
     return launch_status();
 }
 
@@ -407,9 +414,11 @@ int launch_rows(const void* x, int64_t M, int64_t K, int64_t ldx, void* q, void*
 #undef LLMQ_LAUNCH_NCW
         return launch_status();
     }
-#define LLMQ_LAUNCH_NC(NC) \
-    hipLaunchKernelGGL((quant_rows_kernel<DT, MODE, SCALE, NC>), grid, block, 0, st, xp, ldx, K, qp, scale, scale_dtype, aux, n_aux, static_f32, floor)
+#define LLMQ_LAUNCH_NCT(NC, NT) \
+    hipLaunchKernelGGL((quant_rows_kernel<DT, MODE, SCALE, NC, NT>), grid, dim3(NT), 0, st, xp, ldx, K, qp, scale, scale_dtype, aux, n_aux, static_f32, floor)
+#define LLMQ_LAUNCH_NC(NC) LLMQ_LAUNCH_NCT(NC, kThreads)
     if (SCALE != SCALE_ROW) LLMQ_LAUNCH_NC(0);
+    else if (half_blocks(M, K)) LLMQ_LAUNCH_NCT(4, kThreads / 2);
     else if (per_thread <= 1) LLMQ_LAUNCH_NC(1);
     else if (per_thread <= 2) LLMQ_LAUNCH_NC(2);
     else if (per_thread <= 4) LLMQ_LAUNCH_NC(4);

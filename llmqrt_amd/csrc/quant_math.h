@@ -50,6 +50,17 @@ __device__ __forceinline__ float quotient(float x, float s, float inv_s) {
     if (QUOT == Q_DIV_DT || DT == LLMQ_F16) return Lo<DT>::round(x / s);
     return Lo<DT>::round(x * inv_s);
 }
+// the quotients of a pair of elements; the two roundings to the activation dtype share one packed conversion
+template <int DT, int QUOT>
+__device__ __forceinline__ void quotient2(float x0, float x1, float s, float inv_s, float& q0, float& q1) {
+    if (QUOT == Q_DIV_F32) {
+        q0 = x0 / s, q1 = x1 / s;
+        return;
+    }
+    const bool mul = !(QUOT == Q_DIV_DT || DT == LLMQ_F16);
+    const uint32_t p = Lo<DT>::pack2(mul ? x0 * inv_s : x0 / s, mul ? x1 * inv_s : x1 / s);
+    q0 = Lo<DT>::lo_f32(p), q1 = Lo<DT>::hi_f32(p);
+}
 
 // FIN: the caller knows that no quotient can be NaN (the row's absmax, reduced so that a NaN element makes it NaN, is
 // finite, so every element is finite, and the scale is positive): the per-element NaN handling, which then never
@@ -60,12 +71,13 @@ __device__ __forceinline__ uint2 quant8(uint4 raw, float s, float inv_s) {
     float f[8];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        f[2 * i] = Lo<DT>::to_f32((uint16_t)(w[i] & 0xffffu));
-        f[2 * i + 1] = Lo<DT>::to_f32((uint16_t)(w[i] >> 16));
+        float q0, q1;
+        quotient2<DT, QUOT>(Lo<DT>::lo_f32(w[i]), Lo<DT>::hi_f32(w[i]), s, inv_s, q0, q1);
+        f[2 * i] = q0, f[2 * i + 1] = q1;
     }
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        float q = quotient<DT, QUOT>(f[i], s, inv_s);
+        const float q = f[i];
         if (MODE == MODE_I8) {
             f[i] = (!FIN && q != q) ? 0.f : q;  // NaN narrows to 0 (what the reference's cast gives); clamp: see below
         } else {
