@@ -1,4 +1,4 @@
-"""CPU: the SmoothQuant smoothing used by the decoder-layer stack (BASELINE configs[4]).
+"""CPU: the SmoothQuant smoothing used by the decoder-layer stack (the decoder-layer workload of the benchmark contract).
 
 The smoothing formula is not in the reference repository (it ships pre-smoothed checkpoints); it is pinned
 here by what the mathematics fixes: the identity (X / s)(s W)^T = X W^T, the balance point
