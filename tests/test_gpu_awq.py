@@ -125,6 +125,31 @@ def test_gemm_random_shapes(cuda):
         assert rel <= 1e-2, (case, M, N, K, G, rel)
 
 
+def test_gemm_wide_random_sweep_equals_dequantize_then_matmul(cuda):
+    """400 seeded shapes over every path behind awq_gemm_triton (few-token kernel with 1-4 token slabs, streaming kernels,
+    tile kernel, dequantize + fp16 GEMM; groups 32 / 64 / 128; N from 32 to 8000; random 32-bit words, i.e. every nibble
+    value everywhere): the product against the library's own dequantizer (bit-exact against the oracle, above) followed
+    by an fp32 matmul - the equivalence the reference's module relies on when it switches paths at 1024 tokens
+    (nn_models/modules/linear/linear_awq.py:64-65)."""
+    import random
+    from llmqrt_amd.awq_kernels import awq_dequantize_triton, awq_gemm_triton
+    rnd = random.Random(4242)
+    for case in range(400):
+        M = rnd.choice([1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 100, 256, 300, 1024, 1500])
+        G = rnd.choice([128, 128, 128, 64, 32])
+        K = G * rnd.randint(1, 40 if G == 128 else 20)
+        N = 8 * rnd.choice([4, 8, 12, 16, 20, 32, 33, 64, 100, 128, 448, 576, 1000])
+        g = torch.Generator(device=cuda).manual_seed(case)
+        qw = torch.randint(-2**31, 2**31 - 1, (K, N // 8), dtype=torch.int32, device=cuda, generator=g)
+        qz = torch.randint(-2**31, 2**31 - 1, (K // G, N // 8), dtype=torch.int32, device=cuda, generator=g)
+        sc = (torch.rand(K // G, N, device=cuda, generator=g) * 0.02 + 0.001).half()
+        x = torch.randn(M, K, device=cuda, generator=g).half()
+        y = awq_gemm_triton(x, qw, sc, qz, 8)
+        ref = x.float() @ awq_dequantize_triton(qw, sc, qz).float()
+        err = ((y.float() - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
+        assert err <= REL_TOL, (case, M, N, K, G, err)
+
+
 @pytest.mark.parametrize("K", [512, 8320])
 def test_module_paths_agree_around_the_token_threshold(cuda, K):
     """WQLinear_GEMM switches from the fused kernel to dequantize + matmul at a measured token count; one token

@@ -386,6 +386,59 @@ def test_w8a8_random_shapes(cuda):
         assert torch.equal(y2.view(torch.int16), y.view(torch.int16)), (case, M, N, K)
 
 
+_SWEEP_M = [1, 2, 3, 5, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 500, 512, 1000, 1024, 2047, 2048, 2049, 4096,
+            8192]
+_SWEEP_N = [8, 16, 24, 100, 128, 136, 256, 264, 512, 520, 1000, 3584, 4608, 8192, 12345]
+_SWEEP_K16 = [1, 2, 3, 4, 7, 8, 9, 16, 24, 32, 33, 64, 100, 224, 256, 448, 1184]
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_wide_random_sweep_against_fp64_matmul(cuda, fp8):
+    """600 seeded problem sizes per operand type that cross every plan boundary (few-token kernel, every tile shape, K
+    splits, tail split, ragged M / N, K from 16 bytes to 18944): accumulators against an fp64 matmul of the same
+    operands on the GPU (exact for int8: every partial sum is an integer below 2^53; fp8 within the accumulation-window
+    tolerance), outputs against the epilogue formula in fp64, and the launch with an accumulator dump bit-identical
+    to the one without (int8)."""
+    import random
+    from llmqrt_amd.sq_fp8_kernels import cutlass_f8f8bf16_rowwise_sm89, w8a8_int8_linear_bbf16_obf16_per_channel
+    rnd = random.Random(77 + fp8)
+
+    def rel(a, b):
+        return ((a.double() - b).abs().max() / b.abs().max().clamp_min(1e-30)).item()
+    done = 0
+    for case in range(700):
+        M = rnd.choice(_SWEEP_M) if rnd.random() < 0.7 else rnd.randint(1, 3000)
+        N = rnd.choice(_SWEEP_N) if rnd.random() < 0.7 else rnd.randint(1, 9000)
+        K = 16 * (rnd.choice(_SWEEP_K16) if rnd.random() < 0.7 else rnd.randint(1, 600))
+        if M * N > 48 << 20:
+            continue
+        g = torch.Generator(device=cuda).manual_seed(case)
+        bias = torch.randn(N, device=cuda, generator=g).bfloat16()
+        sa = torch.rand(M, 1, device=cuda, generator=g) * 0.05 + 0.001
+        sw = torch.rand(1, N, device=cuda, generator=g) * 0.02 + 0.001
+        if fp8:
+            a = (torch.randn(M, K, device=cuda, generator=g) * 3).to(torch.float8_e4m3fn)
+            b = (torch.randn(N, K, device=cuda, generator=g) * 3).to(torch.float8_e4m3fn)
+            dump = torch.empty(M, N, dtype=torch.float32, device=cuda)
+            y = cutlass_f8f8bf16_rowwise_sm89(a, b.t(), bias, sa, sw, True, _acc_dump=dump)
+            y2 = cutlass_f8f8bf16_rowwise_sm89(a, b.t(), bias, sa, sw, True)
+            acc = a.double() @ b.double().t()
+            assert rel(dump, acc) <= FP8_ACC_TOL, (case, M, N, K)
+        else:
+            a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device=cuda, generator=g)
+            b = torch.randint(-128, 128, (N, K), dtype=torch.int8, device=cuda, generator=g)
+            dump = torch.empty(M, N, dtype=torch.int32, device=cuda)
+            y = w8a8_int8_linear_bbf16_obf16_per_channel(a, b.t(), bias, sa, sw, _acc_dump=dump)
+            y2 = w8a8_int8_linear_bbf16_obf16_per_channel(a, b.t(), bias, sa, sw)
+            acc = a.double() @ b.double().t()
+            assert torch.equal(dump.double(), acc), (case, M, N, K)
+            assert torch.equal(y.view(torch.int16), y2.view(torch.int16)), (case, M, N, K)
+        ref = (acc * sa.double()) * sw.double() + bias.double()
+        assert rel(y, ref) <= REL_TOL and rel(y2, ref) <= REL_TOL, (case, M, N, K)
+        done += 1
+    assert done >= 600
+
+
 def test_w8a8_full_prefill_size_properties(cuda):
     """The largest launch of the benchmark (M = 8192, N = 37888, K = 3584): 48 sampled token rows of the int32
     accumulators against the exact integer GEMM, the fast epilogue equal to the general one on every element,

@@ -11,9 +11,10 @@ from oracle import ref_math as R
 pytestmark = pytest.mark.gpu
 
 INV_RTOL = 5e-7  # ~4 ulp of fp32: summation order + one sqrt + one division
-# the last four take the wavefront-per-row kernels (256 rows or more of at most 1024 elements)
+# (258, 896) .. (257, 520) take the wavefront-per-row kernels (256 rows or more of at most 1024 elements), the last three
+# the half-size blocks with four chunks per thread (256 rows or more of 2056 .. 4096 elements)
 SHAPES = [(1, 896), (16, 896), (7, 3584), (128, 3584), (33, 18944), (3, 8), (5, 24576), (2, 40960),
-          (258, 896), (1027, 1024), (300, 8), (257, 520)]
+          (258, 896), (1027, 1024), (300, 8), (257, 520), (300, 3584), (257, 2056), (256, 4096)]
 
 
 def _inputs(M, K, dtype, seed):

@@ -12,10 +12,11 @@ def _acts(M, K, seed, dtype):
     return W.activations(M, K, seed, dtype=dtype)
 
 
-# the last four take the wavefront-per-row kernels (256 rows or more of at most 1024 elements): ragged row counts,
-# one and two chunks per lane, rows shorter than a wavefront
+# (258, 896) .. (257, 520) take the wavefront-per-row kernels (256 rows or more of at most 1024 elements): ragged row
+# counts, one and two chunks per lane, rows shorter than a wavefront; the last three the half-size blocks with four
+# chunks per thread (256 rows or more of 2056 .. 4096 elements): the shortest and longest such rows and K = 3584
 SHAPES = [(1, 896), (16, 896), (7, 3584), (128, 3584), (33, 18944), (3, 8), (5, 24576), (2, 40960),
-          (258, 896), (1027, 1024), (300, 8), (257, 520)]
+          (258, 896), (1027, 1024), (300, 8), (257, 520), (300, 3584), (257, 2056), (256, 4096)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -191,8 +192,9 @@ def test_sq_per_channel_module_quantizes_its_weight_on_the_gpu(cuda):
 
 # ---- NaN inputs: torch's max / amax propagate a NaN into the scale, so the whole row (per token) or the whole tensor
 # (per tensor) comes out as NaN scale with zero int8 codes / NaN fp8 codes.  (7, 3584): a block per row with the row
-# in registers; (300, 512): a wavefront per row; (3, 24576): a block per row, second pass re-reading the row.
-NAN_SHAPES = [(7, 3584), (300, 512), (3, 24576)]
+# in registers; (300, 512): a wavefront per row; (3, 24576): a block per row, second pass re-reading the row;
+# (260, 3584): half-size blocks with four chunks per thread.
+NAN_SHAPES = [(7, 3584), (300, 512), (3, 24576), (260, 3584)]
 
 
 def _with_nans(M, K, seed, dtype):
