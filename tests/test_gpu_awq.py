@@ -125,6 +125,22 @@ def test_gemm_random_shapes(cuda):
         assert rel <= 1e-2, (case, M, N, K, G, rel)
 
 
+@pytest.mark.parametrize("M", [1, 16, 64, 200])
+def test_gemm_at_a_vocabulary_size_n(cuda, M):
+    """N = 152064 (594 column tiles of the few-token kernel, more blocks than any projection of the benchmark) on every
+    path by token count, against the library's own dequantizer + fp32 matmul."""
+    from llmqrt_amd.awq_kernels import awq_dequantize_triton, awq_gemm_triton
+    K, N, G = 3584, 152064, 128
+    g = torch.Generator(device=cuda).manual_seed(M)
+    qw = torch.randint(-2**31, 2**31 - 1, (K, N // 8), dtype=torch.int32, device=cuda, generator=g)
+    qz = torch.randint(-2**31, 2**31 - 1, (K // G, N // 8), dtype=torch.int32, device=cuda, generator=g)
+    sc = (torch.rand(K // G, N, device=cuda, generator=g) * 0.02 + 0.001).half()
+    x = torch.randn(M, K, device=cuda, generator=g).half()
+    y = awq_gemm_triton(x, qw, sc, qz, 8)
+    ref = x.float() @ awq_dequantize_triton(qw, sc, qz).float()
+    assert ((y.float() - ref).abs().max() / ref.abs().max()).item() <= REL_TOL
+
+
 def test_gemm_wide_random_sweep_equals_dequantize_then_matmul(cuda):
     """400 seeded shapes over every path behind awq_gemm_triton (few-token kernel with 1-4 token slabs, streaming kernels,
     tile kernel, dequantize + fp16 GEMM; groups 32 / 64 / 128; N from 32 to 8000; random 32-bit words, i.e. every nibble

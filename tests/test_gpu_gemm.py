@@ -439,6 +439,40 @@ def test_wide_random_sweep_against_fp64_matmul(cuda, fp8):
     assert done >= 600
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("M,N,K", [(16, 152064, 3584), (300, 152064, 3584), (8, 256, 4194288), (70000, 64, 256)])
+def test_extreme_sizes(cuda, fp8, M, N, K):
+    """A vocabulary-size N, the longest K the entry points accept (row strides below 2^22 bytes) and many more rows than
+    any tile grid the benchmark uses: accumulators against an fp64 matmul on the GPU in blocks of rows (int8 exact)."""
+    from llmqrt_amd.sq_fp8_kernels import cutlass_f8f8bf16_rowwise_sm89, w8a8_int8_linear_bbf16_obf16_per_channel
+    g = torch.Generator(device=cuda).manual_seed(M + N + K)
+    bias = torch.zeros(N, device=cuda, dtype=torch.bfloat16)
+    sa = torch.rand(M, 1, device=cuda, generator=g) * 0.05 + 0.001
+    sw = torch.rand(1, N, device=cuda, generator=g) * 0.02 + 0.001
+    if fp8:
+        a = (torch.randn(M, K, device=cuda, generator=g) * 3).to(torch.float8_e4m3fn)
+        b = (torch.randn(N, K, device=cuda, generator=g) * 3).to(torch.float8_e4m3fn)
+        dump = torch.empty(M, N, dtype=torch.float32, device=cuda)
+        y = cutlass_f8f8bf16_rowwise_sm89(a, b.t(), bias, sa, sw, True, _acc_dump=dump)
+    else:
+        a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device=cuda, generator=g)
+        b = torch.randint(-128, 128, (N, K), dtype=torch.int8, device=cuda, generator=g)
+        dump = torch.empty(M, N, dtype=torch.int32, device=cuda)
+        y = w8a8_int8_linear_bbf16_obf16_per_channel(a, b.t(), bias, sa, sw, _acc_dump=dump)
+    for m0 in range(0, M, 4096):
+        am = a[m0:m0 + 4096].double()
+        for n0 in range(0, N, 16384):
+            acc = am @ b[n0:n0 + 16384].double().t()
+            d = dump[m0:m0 + 4096, n0:n0 + 16384].double()
+            if fp8:
+                assert ((d - acc).abs().max() / acc.abs().max()).item() <= FP8_ACC_TOL, (m0, n0)
+            else:
+                assert torch.equal(d, acc), (m0, n0)
+            ref = (acc * sa[m0:m0 + 4096].double()) * sw[:, n0:n0 + 16384].double()
+            out = y[m0:m0 + 4096, n0:n0 + 16384].double()
+            assert ((out - ref).abs().max() / ref.abs().max()).item() <= REL_TOL, (m0, n0)
+
+
 def test_w8a8_full_prefill_size_properties(cuda):
     """The largest launch of the benchmark (M = 8192, N = 37888, K = 3584): 48 sampled token rows of the int32
     accumulators against the exact integer GEMM, the fast epilogue equal to the general one on every element,
